@@ -16,6 +16,11 @@ from torch.utils.cpp_extension import BuildExtension, CUDAExtension  # noqa: E40
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 OPS = os.path.join(ROOT, "xllm_service_amd", "csrc", "ops")
+HYB = os.path.join(ROOT, "xllm_service_amd", "csrc", "hybrid")
+
+# hipcc only: fp32 math compiles to scalar-lane ops (no packed fp32 forms)
+HIP_FLAGS = ["-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops"]
 
 ext_modules = [
     CUDAExtension(
@@ -38,10 +43,31 @@ ext_modules = [
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],
-            "nvcc": ["-O3", "-std=c++17"],
+            "nvcc": HIP_FLAGS,
+        },
+    ),
+    # hybrid sequence mixers (latent attention, decayed linear attention),
+    # grouped norms and routed experts; bf16 and fp32 activations
+    CUDAExtension(
+        name="xllm_service_amd._ops_hybrid",
+        sources=[
+            os.path.join(HYB, f)
+            for f in ("bindings.cpp", "norms.hip", "latent_attn.hip",
+                      "decay_attn.hip", "moe.hip")
+        ],
+        extra_compile_args={
+            "cxx": ["-O3", "-std=c++17"],
+            "nvcc": HIP_FLAGS,
         },
     ),
 ]
+
+# XLLM_BUILD_EXT=<module name>[,<module name>] builds only those extensions
+# (a worker compiles just what its model needs on first start)
+_only = [n for n in os.environ.get("XLLM_BUILD_EXT", "").split(",") if n]
+if _only:
+    ext_modules = [e for e in ext_modules
+                   if e.name.rsplit(".", 1)[-1] in _only]
 
 setup(
     name="xllm_service_amd",

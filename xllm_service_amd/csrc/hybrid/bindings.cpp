@@ -1,0 +1,297 @@
+// PyTorch bindings for the hybrid-mixer kernels (latent attention, decayed
+// linear attention, grouped norms, routed experts). Shape/dtype validation
+// lives here; activations may be bf16 or fp32, everything the kernels
+// accumulate or carry is fp32.
+#include <hip/hip_runtime.h>
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+
+namespace xllm {
+namespace hyb {
+template <typename TI, typename TO>
+void launch_group_rmsnorm(TO*, const TI*, const float*, float, int, int, int,
+                          long, hipStream_t);
+template <typename TY, typename TG>
+void launch_gated_norm_residual(float*, const TY*, const TG*, const float*,
+                                const float*, const float*, float, float, int,
+                                int, int, long, hipStream_t);
+template <typename T>
+void launch_norm_sigmoid_gate(T*, const float*, const float*, const T*, float,
+                              int, int, long, hipStream_t);
+template <typename T>
+void launch_silu_mul(T*, const T*, long, int, hipStream_t);
+template <typename T>
+void launch_rope_interleaved(T*, const long*, const double*, float, int, int,
+                             int, long, long, int, hipStream_t);
+template <typename T>
+void launch_latent_kv_store(T*, const T*, const float*, float, const long*,
+                            const double*, float, int, const long*, int, int,
+                            int, long, hipStream_t);
+template <typename T>
+void launch_latent_attn(float*, const T*, const T*, const int*, const int*,
+                        const int*, int, int, int, int, int, int, int, float,
+                        long, hipStream_t);
+template <typename T>
+void launch_decay_attn(float*, const T*, const T*, const T*, const float*,
+                       float*, const int*, const int*, const int*, int, int,
+                       int, int, long, long, long, hipStream_t);
+template <typename T>
+void launch_moe_route(int*, float*, const T*, const float*, int, int, int, int,
+                      int, int, long, hipStream_t);
+template <typename T>
+void launch_moe_combine(float*, const T*, const int*, const float*, long, int,
+                        int, hipStream_t);
+}  // namespace hyb
+}  // namespace xllm
+
+namespace {
+using torch::Tensor;
+using bf = unsigned short;
+namespace hy = xllm::hyb;
+
+inline hipStream_t cur() { return at::hip::getCurrentHIPStream().stream(); }
+inline bool is_bf16(const Tensor& t) { return t.dtype() == torch::kBFloat16; }
+inline bool is_f32(const Tensor& t) { return t.dtype() == torch::kFloat; }
+
+#define CHK_ACT(t)                                                       \
+  TORCH_CHECK((t).is_cuda() && (is_bf16(t) || is_f32(t)),                \
+              #t " must be a bf16/fp32 GPU tensor");                     \
+  TORCH_CHECK((t).stride(-1) == 1, #t " innermost dim must be contiguous")
+#define CHK_F32C(t)                                                      \
+  TORCH_CHECK((t).is_cuda() && is_f32(t) && (t).is_contiguous(),         \
+              #t " must be a contiguous fp32 GPU tensor")
+#define CHK_I32C(t)                                                      \
+  TORCH_CHECK((t).is_cuda() && (t).dtype() == torch::kInt &&             \
+              (t).is_contiguous(), #t " must be contiguous int32 on GPU")
+#define CHK_I64C(t)                                                      \
+  TORCH_CHECK((t).is_cuda() && (t).dtype() == torch::kLong &&            \
+              (t).is_contiguous(), #t " must be contiguous int64 on GPU")
+
+template <typename T> T* ptr(const Tensor& t) {
+  return reinterpret_cast<T*>(t.data_ptr());
+}
+
+// out [rows, width] contiguous (bf16|fp32), x 2-D with unit inner stride
+void group_rmsnorm(Tensor out, Tensor x, Tensor w, double eps, long groups) {
+  CHK_ACT(out); CHK_ACT(x); CHK_F32C(w);
+  TORCH_CHECK(x.dim() == 2 && out.dim() == 2 && out.is_contiguous());
+  const int rows = x.size(0), width = x.size(1);
+  TORCH_CHECK(out.size(0) == rows && out.size(1) == width &&
+              w.numel() == width && groups >= 1 && width % groups == 0);
+  const long xs = x.stride(0);
+  auto st = cur();
+  if (is_f32(x) && is_f32(out))
+    hy::launch_group_rmsnorm<float, float>(ptr<float>(out), ptr<float>(x), ptr<float>(w), eps, rows, width, groups, xs, st);
+  else if (is_f32(x))
+    hy::launch_group_rmsnorm<float, bf>(ptr<bf>(out), ptr<float>(x), ptr<float>(w), eps, rows, width, groups, xs, st);
+  else if (is_f32(out))
+    hy::launch_group_rmsnorm<bf, float>(ptr<float>(out), ptr<bf>(x), ptr<float>(w), eps, rows, width, groups, xs, st);
+  else
+    hy::launch_group_rmsnorm<bf, bf>(ptr<bf>(out), ptr<bf>(x), ptr<float>(w), eps, rows, width, groups, xs, st);
+}
+
+void gated_norm_residual(Tensor res, Tensor y, Tensor gate,
+                         c10::optional<Tensor> bias, Tensor w, Tensor ls,
+                         double mult, double eps, long groups) {
+  CHK_F32C(res); CHK_ACT(y); CHK_ACT(gate); CHK_F32C(w); CHK_F32C(ls);
+  TORCH_CHECK(res.dim() == 2 && y.dim() == 2 && gate.dim() == 2 &&
+              y.is_contiguous());
+  const int rows = res.size(0), width = res.size(1);
+  TORCH_CHECK(y.size(0) == rows && y.size(1) == width &&
+              gate.size(0) == rows && gate.size(1) == width &&
+              w.numel() == width && ls.numel() == width &&
+              groups >= 1 && width % groups == 0);
+  const float* b = nullptr;
+  if (bias.has_value()) {
+    CHK_F32C(*bias);
+    TORCH_CHECK(bias->numel() == width);
+    b = ptr<float>(*bias);
+  }
+  const long gs = gate.stride(0);
+  auto st = cur();
+  if (is_f32(y) && is_f32(gate))
+    hy::launch_gated_norm_residual<float, float>(ptr<float>(res), ptr<float>(y), ptr<float>(gate), b, ptr<float>(w), ptr<float>(ls), mult, eps, rows, width, groups, gs, st);
+  else if (is_f32(y))
+    hy::launch_gated_norm_residual<float, bf>(ptr<float>(res), ptr<float>(y), ptr<bf>(gate), b, ptr<float>(w), ptr<float>(ls), mult, eps, rows, width, groups, gs, st);
+  else {
+    TORCH_CHECK(is_bf16(gate), "bf16 y needs a bf16 gate");
+    hy::launch_gated_norm_residual<bf, bf>(ptr<float>(res), ptr<bf>(y), ptr<bf>(gate), b, ptr<float>(w), ptr<float>(ls), mult, eps, rows, width, groups, gs, st);
+  }
+}
+
+void norm_sigmoid_gate(Tensor out, Tensor o, c10::optional<Tensor> w,
+                       Tensor gate, double eps) {
+  CHK_ACT(out); CHK_F32C(o); CHK_ACT(gate);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && gate.dim() == 2);
+  const int rows = out.size(0), n = out.size(1);
+  TORCH_CHECK(o.numel() == (long)rows * n && gate.size(0) == rows &&
+              gate.size(1) == n && gate.dtype() == out.dtype());
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    CHK_F32C(*w);
+    TORCH_CHECK(w->numel() == n);
+    wp = ptr<float>(*w);
+  }
+  if (is_f32(out))
+    hy::launch_norm_sigmoid_gate<float>(ptr<float>(out), ptr<float>(o), wp, ptr<float>(gate), eps, rows, n, gate.stride(0), cur());
+  else
+    hy::launch_norm_sigmoid_gate<bf>(ptr<bf>(out), ptr<float>(o), wp, ptr<bf>(gate), eps, rows, n, gate.stride(0), cur());
+}
+
+void silu_mul(Tensor out, Tensor x) {
+  CHK_ACT(out); CHK_ACT(x);
+  TORCH_CHECK(out.is_contiguous() && x.is_contiguous() &&
+              out.dtype() == x.dtype());
+  const int F = out.size(-1);
+  TORCH_CHECK(x.size(-1) == 2 * F && x.numel() == 2 * out.numel());
+  const long rows = out.numel() / F;
+  if (is_f32(x)) hy::launch_silu_mul<float>(ptr<float>(out), ptr<float>(x), rows, F, cur());
+  else hy::launch_silu_mul<bf>(ptr<bf>(out), ptr<bf>(x), rows, F, cur());
+}
+
+// x [T, H, D] view (unit inner stride); rotates x[..., off:off+rot_dims]
+void rope_interleaved(Tensor x, Tensor pos, Tensor inv_freq, double mscale,
+                      long off, long rot_dims) {
+  CHK_ACT(x); CHK_I64C(pos);
+  TORCH_CHECK(inv_freq.is_cuda() && inv_freq.dtype() == torch::kDouble &&
+              inv_freq.is_contiguous());
+  TORCH_CHECK(x.dim() == 3 && pos.numel() == x.size(0));
+  TORCH_CHECK(rot_dims % 2 == 0 && off >= 0 && off + rot_dims <= x.size(2) &&
+              inv_freq.numel() == rot_dims / 2);
+  const int T = x.size(0), H = x.size(1);
+  if (is_f32(x))
+    hy::launch_rope_interleaved<float>(ptr<float>(x), ptr<long>(pos), ptr<double>(inv_freq), mscale, T, H, rot_dims / 2, x.stride(0), x.stride(1), off, cur());
+  else
+    hy::launch_rope_interleaved<bf>(ptr<bf>(x), ptr<long>(pos), ptr<double>(inv_freq), mscale, T, H, rot_dims / 2, x.stride(0), x.stride(1), off, cur());
+}
+
+// cache [blocks, bs, r+rd]; dkv [T, r+rd] row view
+void latent_kv_store(Tensor cache, Tensor dkv, Tensor norm_w, double eps,
+                     Tensor pos, Tensor inv_freq, double mscale,
+                     long rot_dims, Tensor slots, long kv_rank) {
+  CHK_ACT(cache); CHK_ACT(dkv); CHK_F32C(norm_w); CHK_I64C(pos);
+  CHK_I64C(slots);
+  TORCH_CHECK(cache.is_contiguous() && cache.dim() == 3 && dkv.dim() == 2 &&
+              cache.dtype() == dkv.dtype());
+  TORCH_CHECK(inv_freq.is_cuda() && inv_freq.dtype() == torch::kDouble &&
+              inv_freq.is_contiguous());
+  const int T = dkv.size(0), W = dkv.size(1);
+  const int r = kv_rank, rd = W - r;
+  TORCH_CHECK(cache.size(2) == W && r > 0 && rd >= 0 && rot_dims <= rd &&
+              rot_dims % 2 == 0 && norm_w.numel() == r &&
+              inv_freq.numel() == rot_dims / 2 && pos.numel() == T &&
+              slots.numel() == T);
+  if (is_f32(dkv))
+    hy::launch_latent_kv_store<float>(ptr<float>(cache), ptr<float>(dkv), ptr<float>(norm_w), eps, ptr<long>(pos), ptr<double>(inv_freq), mscale, rot_dims, ptr<long>(slots), T, r, rd, dkv.stride(0), cur());
+  else
+    hy::launch_latent_kv_store<bf>(ptr<bf>(cache), ptr<bf>(dkv), ptr<float>(norm_w), eps, ptr<long>(pos), ptr<double>(inv_freq), mscale, rot_dims, ptr<long>(slots), T, r, rd, dkv.stride(0), cur());
+}
+
+// out fp32 [T, H, r]; q [T, H, r+rd] contiguous; cu_q None => decode
+void latent_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables,
+                 c10::optional<Tensor> cu_q, Tensor seq_lens, double scale,
+                 long kv_rank) {
+  CHK_F32C(out); CHK_ACT(q); CHK_ACT(cache); CHK_I32C(block_tables);
+  CHK_I32C(seq_lens);
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && cache.is_contiguous() &&
+              cache.dim() == 3 && q.dtype() == cache.dtype() &&
+              block_tables.dim() == 2);
+  const int T = q.size(0), H = q.size(1), W = q.size(2);
+  const int r = kv_rank;
+  TORCH_CHECK(cache.size(2) == W && r > 0 && r <= W && r <= 64 * 16,
+              "latent width mismatch or kv_rank > 1024");
+  TORCH_CHECK(out.numel() == (long)T * H * r);
+  const int n_seqs = seq_lens.numel();
+  TORCH_CHECK(block_tables.size(0) == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  const int nw = H < 4 ? H : 4;
+  TORCH_CHECK((size_t)nw * W * 4 <= 64 * 1024, "query row too wide for LDS");
+  if (is_f32(q))
+    hy::launch_latent_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, H, r, W - r, cache.size(1), block_tables.size(1), scale, q.stride(0), cur());
+  else
+    hy::launch_latent_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, H, r, W - r, cache.size(1), block_tables.size(1), scale, q.stride(0), cur());
+}
+
+// out fp32 [T, H, Dv]; q,k [T, H*D] / v [T, H*Dv] row views (pre-activation)
+// state fp32 [slots, H, D, Dv]; cu_q None => one token per sequence
+void decay_attn(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
+                Tensor state, Tensor slots, c10::optional<Tensor> cu_q,
+                Tensor ctx_lens) {
+  CHK_F32C(out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_F32C(decay);
+  CHK_F32C(state); CHK_I32C(slots); CHK_I32C(ctx_lens);
+  TORCH_CHECK(state.dim() == 4 && q.dim() == 2 && k.dim() == 2 &&
+              v.dim() == 2 && q.dtype() == k.dtype() && q.dtype() == v.dtype());
+  const int H = state.size(1), D = state.size(2), Dv = state.size(3);
+  const int T = q.size(0);
+  TORCH_CHECK(q.size(1) == H * D && k.size(1) == H * D && v.size(1) == H * Dv &&
+              k.size(0) == T && v.size(0) == T && decay.numel() == H);
+  TORCH_CHECK(D <= 256, "key dim > 256 unsupported");
+  TORCH_CHECK(out.numel() == (long)T * H * Dv);
+  const int n_seqs = slots.numel();
+  TORCH_CHECK(ctx_lens.numel() == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  if (is_f32(q))
+    hy::launch_decay_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), cur());
+  else
+    hy::launch_decay_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), cur());
+}
+
+void moe_route(Tensor ids, Tensor wts, Tensor h, Tensor wr, long top,
+               long n_groups, long keep) {
+  CHK_I32C(ids); CHK_F32C(wts); CHK_ACT(h); CHK_F32C(wr);
+  TORCH_CHECK(h.dim() == 2 && wr.dim() == 2);
+  const int T = h.size(0), width = h.size(1), E = wr.size(0);
+  TORCH_CHECK(wr.size(1) == width && ids.numel() == (long)T * top &&
+              wts.numel() == (long)T * top);
+  TORCH_CHECK(top >= 1 && top <= E && n_groups >= 1 && E % n_groups == 0 &&
+              keep >= 1 && keep <= n_groups &&
+              keep * (E / n_groups) >= top, "bad routing constants");
+  TORCH_CHECK((2 * E + n_groups) * 4 <= 64 * 1024, "too many experts");
+  if (is_f32(h))
+    hy::launch_moe_route<float>(ptr<int>(ids), ptr<float>(wts), ptr<float>(h), ptr<float>(wr), T, width, E, top, n_groups, keep, h.stride(0), cur());
+  else
+    hy::launch_moe_route<bf>(ptr<int>(ids), ptr<float>(wts), ptr<bf>(h), ptr<float>(wr), T, width, E, top, n_groups, keep, h.stride(0), cur());
+}
+
+// out fp32 [T, width]; y [R, width] contiguous; rows int32 [T, top] < R
+void moe_combine(Tensor out, Tensor y, Tensor rows, Tensor wts) {
+  CHK_F32C(out); CHK_ACT(y); CHK_I32C(rows); CHK_F32C(wts);
+  TORCH_CHECK(y.is_contiguous() && out.dim() == 2 && rows.dim() == 2);
+  const long T = out.size(0);
+  const int width = out.size(1), top = rows.size(1);
+  TORCH_CHECK(rows.size(0) == T && wts.numel() == T * top &&
+              y.size(-1) == width);
+  if (is_f32(y))
+    hy::launch_moe_combine<float>(ptr<float>(out), ptr<float>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, cur());
+  else
+    hy::launch_moe_combine<bf>(ptr<float>(out), ptr<bf>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, cur());
+}
+
+}  // namespace
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("group_rmsnorm", &group_rmsnorm);
+  m.def("gated_norm_residual", &gated_norm_residual);
+  m.def("norm_sigmoid_gate", &norm_sigmoid_gate);
+  m.def("silu_mul", &silu_mul);
+  m.def("rope_interleaved", &rope_interleaved);
+  m.def("latent_kv_store", &latent_kv_store);
+  m.def("latent_attn", &latent_attn);
+  m.def("decay_attn", &decay_attn);
+  m.def("moe_route", &moe_route);
+  m.def("moe_combine", &moe_combine);
+}

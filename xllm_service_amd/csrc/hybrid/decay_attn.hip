@@ -1,0 +1,125 @@
+// Decayed linear attention with a carried recurrent state.
+//
+//   S_t = decay_h * S_{t-1} + k_t v_t^T        (S is [D, Dv] per head, fp32)
+//   o_t = S_t^T q_t
+// with q, k, v = silu(projection), the activation fused here. The state
+// lives in a slot pool [slots, H, D, Dv]; a sequence with ctx_len == 0 starts
+// from zero whatever its slot held before.
+//
+// One workgroup per (sequence, head, 16-column slice of Dv): the columns of S
+// are independent, so slices never talk to each other. Thread (j, r) owns the
+// rows i = r, r+16, ... of column j; a token's output column is the sum over
+// the 16 threads sharing j (a 16-lane shuffle reduction). Tokens are staged
+// through LDS 16 at a time.
+#include "hybrid_common.h"
+
+namespace xllm {
+namespace hyb {
+
+constexpr int DA_VS = 16;      // value columns per workgroup
+constexpr int DA_R = 16;       // row groups (threads per column)
+constexpr int DA_TC = 16;      // tokens staged per LDS fill
+constexpr int DA_MAXM = 16;    // D <= DA_R * DA_MAXM = 256
+
+template <typename T>
+__global__ void __launch_bounds__(256) decay_attn_kernel(
+    float* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k,
+    const T* __restrict__ v, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ slots,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int heads,
+    int D, int Dv, long q_stride, long k_stride, long v_stride) {
+  extern __shared__ float smem[];
+  float* qs = smem;                       // [TC][D]
+  float* ks = qs + DA_TC * D;             // [TC][D]
+  float* vs = ks + DA_TC * D;             // [TC][VS]
+
+  const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * DA_VS;
+  const int tid = threadIdx.x;
+  const int j = tid / DA_R, r = tid % DA_R;
+  const int col = v0 + j;
+  const bool col_ok = col < Dv;
+  const int t0 = cu_q ? cu_q[s] : s;
+  const int t1 = cu_q ? cu_q[s + 1] : s + 1;
+  const int slot = slots[s];
+  const float dec = decay[h];
+  const int M = (D + DA_R - 1) / DA_R;
+
+  float S[DA_MAXM];
+#pragma unroll
+  for (int m = 0; m < DA_MAXM; ++m) S[m] = 0.f;
+  float* sp = (slot >= 0)
+      ? state + (((long)slot * heads + h) * D) * (long)Dv : nullptr;
+  if (sp && ctx_lens[s] > 0 && col_ok) {
+#pragma unroll
+    for (int m = 0; m < DA_MAXM; ++m) {
+      const int i = r + DA_R * m;
+      if (m < M && i < D) S[m] = sp[(long)i * Dv + col];
+    }
+  }
+
+  for (int tb = t0; tb < t1; tb += DA_TC) {
+    const int nt = min(DA_TC, t1 - tb);
+    __syncthreads();                      // previous tile fully consumed
+    for (int idx = tid; idx < nt * D; idx += 256) {
+      const int tt = idx / D, i = idx - tt * D;
+      const long row = tb + tt;
+      qs[idx] = IO<T>::rnd(siluf_(IO<T>::ld(q + row * q_stride + h * D + i)));
+      ks[idx] = IO<T>::rnd(siluf_(IO<T>::ld(k + row * k_stride + h * D + i)));
+    }
+    for (int idx = tid; idx < nt * DA_VS; idx += 256) {
+      const int tt = idx / DA_VS, jj = idx - tt * DA_VS;
+      const long row = tb + tt;
+      vs[idx] = (v0 + jj < Dv)
+          ? IO<T>::rnd(siluf_(IO<T>::ld(v + row * v_stride + h * Dv + v0 + jj)))
+          : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vj = vs[tt * DA_VS + j];
+      float o = 0.f;
+#pragma unroll
+      for (int m = 0; m < DA_MAXM; ++m) {
+        const int i = r + DA_R * m;
+        if (m < M && i < D) {
+          S[m] = dec * S[m] + ks[tt * D + i] * vj;
+          o += S[m] * qs[tt * D + i];
+        }
+      }
+      o = group_reduce_sum<DA_R>(o);
+      if (r == 0 && col_ok)
+        out[((long)(tb + tt) * heads + h) * Dv + col] = o;
+    }
+  }
+  if (sp && col_ok) {
+#pragma unroll
+    for (int m = 0; m < DA_MAXM; ++m) {
+      const int i = r + DA_R * m;
+      if (m < M && i < D) sp[(long)i * Dv + col] = S[m];
+    }
+  }
+}
+
+template <typename T>
+void launch_decay_attn(float* out, const T* q, const T* k, const T* v,
+                       const float* decay, float* state, const int* slots,
+                       const int* cu_q, const int* ctx_lens, int n_seqs,
+                       int heads, int D, int Dv, long q_stride, long k_stride,
+                       long v_stride, hipStream_t st) {
+  if (n_seqs == 0) return;
+  dim3 grid(n_seqs, heads, (Dv + DA_VS - 1) / DA_VS);
+  const size_t lds = (size_t)(2 * DA_TC * D + DA_TC * DA_VS) * sizeof(float);
+  hipLaunchKernelGGL((decay_attn_kernel<T>), grid, dim3(256), lds, st, out, q,
+                     k, v, decay, state, slots, cu_q, ctx_lens, heads, D, Dv,
+                     q_stride, k_stride, v_stride);
+}
+
+#define INST_DA(T)                                                            \
+  template void launch_decay_attn<T>(                                         \
+      float*, const T*, const T*, const T*, const float*, float*, const int*, \
+      const int*, const int*, int, int, int, int, long, long, long,           \
+      hipStream_t);
+INST_DA(float)
+INST_DA(unsigned short)
+
+}  // namespace hyb
+}  // namespace xllm

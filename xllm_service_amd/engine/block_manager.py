@@ -161,6 +161,19 @@ class BlockManager:
         blk = seq.block_table[pos // self.block_size]
         return blk * self.block_size + pos % self.block_size
 
+    def ensure_capacity(self, seq: Sequence, num_tokens: int) -> bool:
+        """Grow seq.block_table (unhashed blocks) to hold num_tokens tokens;
+        False, with nothing taken, when the pool cannot cover it."""
+        need = ((num_tokens + self.block_size - 1) // self.block_size
+                - len(seq.block_table))
+        if need > self.num_free:
+            return False
+        for _ in range(max(need, 0)):
+            blk = self._pop_free()
+            self.ref_count[blk] = 1
+            seq.block_table.append(blk)
+        return True
+
     def free(self, seq: Sequence):
         for blk in seq.block_table:
             self._decref(blk)

@@ -17,8 +17,9 @@ from xllm_service_amd.models.registry import create_model
 from .block_manager import BlockManager
 from .model_runner import BLOCK_SIZE, ModelRunner
 from .sampling import SamplingParams
-from .scheduler import EngineScheduler
+from .scheduler import EngineScheduler, ScheduledPrefill, StepPlan
 from .sequence import Sequence, SeqStatus
+from .state_manager import StateSlotManager
 
 
 @dataclass
@@ -98,7 +99,9 @@ class LLMEngine:
                  ssd_swap_dir: Optional[str] = None,
                  tp_size: int = 1,
                  load_state_path: Optional[str] = None,
+                 state_slots: Optional[int] = None,
                  seed: int = 0):
+        # model_name: a preset, or a folder holding config.json + safetensors
         self.cfg: ModelConfig = get_config(model_name)
         # tensor parallelism: every rank of the TP group builds its shard;
         # rank 0 drives scheduling, followers replay broadcast batches
@@ -128,25 +131,47 @@ class LLMEngine:
                 full_sd = shard_llama_state_dict(full_sd, self.cfg, tp_size,
                                                  ps.tp_rank())
             self.model.load_state_dict(full_sd)
+        elif getattr(self.cfg, "model_dir", None):
+            from xllm_service_amd.models.loader import load_model_dir_tensors
+            self.model.load_weights(
+                load_model_dir_tensors(self.cfg.model_dir))
         else:
             self.model.random_init(seed)
         self.model = self.model.eval()
 
         n_kv_local = getattr(self.model, "local_kv_heads", self.cfg.num_kv_heads)
+        specs = ModelRunner.specs_for(self.model, self.cfg)
+        custom_cache = hasattr(self.model, "cache_specs")
+        from .cache_spec import needs_state_slots
+        # recurrent-state layers: one slot per live sequence. Such a state
+        # cannot be rebuilt from shared prefix blocks, so prefix reuse is
+        # off for these models.
+        self.state_manager: Optional[StateSlotManager] = None
+        num_state_slots = 0
+        if needs_state_slots(specs):
+            num_state_slots = state_slots or min(max_num_seqs, 256)
+            self.state_manager = StateSlotManager(num_state_slots)
+            max_num_seqs = min(max_num_seqs, num_state_slots)
+            enable_prefix_caching = False
+        dtype_bytes = 2 if dtype == torch.bfloat16 else 4
         num_blocks = ModelRunner.kv_cache_blocks_for(
             self.cfg, self.device, n_kv_local,
             gpu_memory_utilization=gpu_memory_utilization,
-            dtype_bytes=2 if dtype == torch.bfloat16 else 4,
-            max_blocks=max_kv_blocks)
+            dtype_bytes=dtype_bytes,
+            max_blocks=max_kv_blocks, specs=specs,
+            num_state_slots=num_state_slots)
         self.block_manager = BlockManager(num_blocks, BLOCK_SIZE,
                                           enable_prefix_caching)
         # host-DRAM KV tier ("dram" in the reference's hbm/dram/ssd cache
         # tiers): preempted sequences swap out instead of recomputing
+        # (models with their own cache layout recompute instead)
         n_kv = n_kv_local
-        per_block_bytes = (2 * n_kv * BLOCK_SIZE * self.cfg.head_dim *
-                           (2 if dtype == torch.bfloat16 else 4) *
-                           self.cfg.num_layers)
+        per_block_bytes = max(sum(sp.block_bytes(BLOCK_SIZE, dtype_bytes)
+                                  for sp in specs), 1)
         num_cpu_blocks = max((swap_space_mb << 20) // per_block_bytes, 0)
+        if custom_cache:
+            num_cpu_blocks = 0
+            ssd_swap_dir = None
         self.cpu_block_manager = (
             BlockManager(num_cpu_blocks, BLOCK_SIZE,
                          enable_prefix_caching=False)
@@ -163,7 +188,8 @@ class LLMEngine:
             max_batched_tokens=max_batched_tokens,
             prefill_hold_ms=prefill_hold_ms,
             swap_out=self._swap_out if has_swap else None,
-            swap_in=self._swap_in if has_swap else None)
+            swap_in=self._swap_in if has_swap else None,
+            state_manager=self.state_manager)
         if has_swap:
             self.scheduler.free_cpu_blocks = self._free_cpu_blocks
         self.max_model_len = min(max_model_len, self.cfg.max_position)
@@ -172,7 +198,8 @@ class LLMEngine:
                                   num_blocks, dtype=dtype,
                                   enable_graphs=enable_graphs,
                                   max_model_len=max_model_len,
-                                  max_graph_batch=min(max_num_seqs, 256))
+                                  max_graph_batch=min(max_num_seqs, 256),
+                                  num_state_slots=num_state_slots)
         if self.cpu_block_manager:
             self.runner.alloc_cpu_caches(self.cpu_block_manager.num_blocks)
         if self.device.type == "cuda":
@@ -504,31 +531,105 @@ class LLMEngine:
         self.stats.kv_usage = self.block_manager.usage()
         return pre + outputs
 
+    # ---- teacher-forced scoring --------------------------------------------
+    def score_step(self, entries, finished=()) -> torch.Tensor:
+        """Feed given tokens instead of sampled ones and return logits.
+
+        entries: [(request_id, token_ids, want)] — each request's NEXT
+        tokens, continuing from whatever its cache/state holds (a request
+        is admitted at its first entry), and the indices among these tokens
+        whose logits are wanted. All entries form one batch through the same
+        runner step as generation: multi-token entries are prefill chunks,
+        a single token of a request that already has context is a decode
+        row. Returns fp32 logits [sum(len(want)), vocab] on the CPU, in
+        entry order then `want` order. Requests named in `finished` give
+        their blocks and state slot back after the step.
+        """
+        plan = StepPlan()
+        bm = self.block_manager
+        placed = []                      # (is_decode, index, want)
+        for rid, toks, want in entries:
+            toks = list(toks)
+            if not toks:
+                raise ValueError(f"{rid}: empty entry")
+            seq = self.seqs.get(rid)
+            if seq is None:
+                seq = Sequence(request_id=rid, prompt_token_ids=[],
+                               params=SamplingParams(max_tokens=0))
+                seq.status = SeqStatus.RUNNING
+                if self.state_manager is not None:
+                    self.state_manager.allocate(seq)
+                self.seqs[rid] = seq
+            start = seq.prompt_len
+            if start + len(toks) > self.max_model_len:
+                raise ValueError(f"{rid}: exceeds max_model_len")
+            seq.prompt_token_ids.extend(toks)
+            if len(toks) == 1 and start > 0:
+                if not bm.can_append(seq):
+                    raise RuntimeError("KV block pool exhausted")
+                placed.append((True, len(plan.decodes), list(want)))
+                plan.decodes.append(seq)
+            else:
+                if not bm.ensure_capacity(seq, start + len(toks)):
+                    raise RuntimeError("KV block pool exhausted")
+                placed.append((False, len(plan.prefills), list(want)))
+                plan.prefills.append(ScheduledPrefill(seq, start, len(toks)))
+        cu = [0]
+        for sp in plan.prefills:
+            cu.append(cu[-1] + sp.chunk_len)
+        rows: List[int] = []
+        for is_dec, i, want in placed:
+            if is_dec:
+                if any(w != 0 for w in want):
+                    raise ValueError("decode entry: want must be [0]")
+                rows.extend(cu[-1] + i for _ in want)
+            else:
+                n = plan.prefills[i].chunk_len
+                if any(not 0 <= w < n for w in want):
+                    raise ValueError("want index outside the entry")
+                rows.extend(cu[i] + w for w in want)
+        logits = self.runner.score(plan, bm, rows)
+        for sp in plan.prefills:
+            sp.seq.num_computed_tokens += sp.chunk_len
+        for seq in plan.decodes:
+            seq.num_computed_tokens += 1
+        for rid in finished:
+            self.release_scored(rid)
+        self.stats.steps += 1
+        return logits.cpu()
+
+    def release_scored(self, request_id: str) -> None:
+        seq = self.seqs.pop(request_id, None)
+        if seq is None:
+            return
+        self.block_manager.free(seq)
+        if self.state_manager is not None:
+            self.state_manager.free(seq)
+        if self.runner.graph_runner is not None:
+            self.runner.graph_runner.forget(request_id)
+
     def export_block_bytes(self, block_ids: List[int]) -> bytes:
         """Serialize KV blocks (all layers, k then v) — the DRAM/RPC
         migration transport (CPU path + cross-node fallback; the same-node
         GPU path is xGMI P2P in engine/kv_migration.py)."""
         idx = torch.tensor(block_ids, dtype=torch.long, device=self.device)
         parts = []
-        for (kc, vc) in self.runner.kv_caches:
-            for c in (kc, vc):
-                t = c.index_select(0, idx).contiguous()
-                parts.append(t.view(torch.uint8).cpu().numpy().tobytes())
+        for c in self.runner.paged_tensors():
+            t = c.index_select(0, idx).contiguous()
+            parts.append(t.view(torch.uint8).cpu().numpy().tobytes())
         return b"".join(parts)
 
     def import_block_bytes(self, block_ids: List[int], data: bytes) -> None:
         import numpy as np
         idx = torch.tensor(block_ids, dtype=torch.long, device=self.device)
-        kc0 = self.runner.kv_caches[0][0]
-        per = len(block_ids) * kc0[0].numel() * kc0.element_size()
         off = 0
-        for (kc, vc) in self.runner.kv_caches:
-            for c in (kc, vc):
-                raw = np.frombuffer(data, dtype=np.uint8, count=per, offset=off)
-                t = torch.from_numpy(raw.copy()).view(c.dtype).reshape(
-                    len(block_ids), *c.shape[1:])
-                c[idx] = t.to(self.device)
-                off += per
+        for c in self.runner.paged_tensors():
+            per = len(block_ids) * c[0].numel() * c.element_size()
+            raw = np.frombuffer(data, dtype=np.uint8, count=per, offset=off)
+            t = torch.from_numpy(raw.copy()).view(c.dtype).reshape(
+                len(block_ids), *c.shape[1:])
+            c[idx] = t.to(self.device)
+            off += per
 
     def follower_loop(self) -> None:
         """TP ranks > 0: replay broadcast batches until rank 0 stops."""

@@ -55,12 +55,15 @@ class DecodeGraphRunner:
             seq_lens=torch.full((bs,), 16, dtype=torch.int32, device=dev),
             block_tables=torch.zeros(bs, self.max_blocks, dtype=torch.int32,
                                      device=dev),
+            # recurrent-state slot per row; -1 (padding) touches no state
+            state_slots=torch.full((bs,), -1, dtype=torch.int32, device=dev),
         )
         meta = AttnMetadata(
             num_prefill_tokens=0, num_decode_tokens=bs,
             slot_mapping=static["slot_mapping"],
             decode_seq_lens=static["seq_lens"],
-            decode_block_tables=static["block_tables"])
+            decode_block_tables=static["block_tables"],
+            decode_state_slots=static["state_slots"])
 
         def fwd():
             hidden = self.model(static["input_ids"], static["positions"],
@@ -88,6 +91,8 @@ class DecodeGraphRunner:
                                 pin_memory=True),
             block_tables=torch.zeros(bs, self.max_blocks, dtype=torch.int32,
                                      pin_memory=True),
+            state_slots=torch.full((bs,), -1, dtype=torch.int32,
+                                   pin_memory=True),
         )
 
     # ------------------------------------------------------------------ run
@@ -117,7 +122,8 @@ class DecodeGraphRunner:
     @torch.inference_mode()
     def run(self, input_ids: np.ndarray, positions: np.ndarray,
             slots: np.ndarray, seq_lens: np.ndarray,
-            bt_rows: List[np.ndarray]) -> torch.Tensor:
+            bt_rows: List[np.ndarray],
+            state_slots: Optional[np.ndarray] = None) -> torch.Tensor:
         n = len(input_ids)
         bs = self.bucket_for(n)
         graph, static, logits = self.graphs[bs]
@@ -132,6 +138,12 @@ class DecodeGraphRunner:
         if n < bs:
             pin["seq_lens"].numpy()[n:bs] = 16
         np.stack(bt_rows, out=pin["block_tables"].numpy()[:n])
+        if state_slots is not None:
+            ss = pin["state_slots"].numpy()
+            ss[:n] = state_slots
+            ss[n:bs] = -1
+            static["state_slots"].copy_(pin["state_slots"],
+                                        non_blocking=True)
         static["input_ids"].copy_(pin["i64"][0], non_blocking=True)
         static["positions"].copy_(pin["i64"][1], non_blocking=True)
         static["slot_mapping"].copy_(pin["i64"][2], non_blocking=True)

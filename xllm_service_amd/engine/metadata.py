@@ -33,6 +33,13 @@ class AttnMetadata:
     decode_seq_lens: Optional[torch.Tensor] = None    # [n_decode] int32
     decode_block_tables: Optional[torch.Tensor] = None
 
+    # recurrent-state layers: tokens already folded into each sequence's
+    # state before this step, and the state slot it owns (-1 = none: the
+    # sequence runs from a zero state and stores nothing)
+    prefill_ctx_lens: Optional[torch.Tensor] = None      # [n_prefill] int32
+    prefill_state_slots: Optional[torch.Tensor] = None   # [n_prefill] int32
+    decode_state_slots: Optional[torch.Tensor] = None    # [n_decode] int32
+
     @property
     def num_tokens(self) -> int:
         return self.num_prefill_tokens + self.num_decode_tokens

@@ -13,6 +13,8 @@ import torch
 from xllm_service_amd import ops
 from xllm_service_amd.models.config import ModelConfig
 
+from .cache_spec import (PagedKV, PagedLatent, RecurrentState, SharedCache,
+                         default_specs, needs_state_slots)
 from .metadata import AttnMetadata
 from .scheduler import StepPlan
 from .sequence import Sequence
@@ -24,7 +26,7 @@ class ModelRunner:
     def __init__(self, model, cfg: ModelConfig, device: torch.device,
                  num_blocks: int, dtype=torch.bfloat16,
                  enable_graphs: bool = True, max_model_len: int = 4096,
-                 max_graph_batch: int = 256):
+                 max_graph_batch: int = 256, num_state_slots: int = 0):
         self.model = model
         self.cfg = cfg
         self.device = device
@@ -33,15 +35,51 @@ class ModelRunner:
         self.graph_runner = None
         self._graph_opts = (enable_graphs and device.type == "cuda",
                             max_model_len, max_graph_batch)
-        n_kv = model.local_kv_heads if hasattr(model, "local_kv_heads") else cfg.num_kv_heads
-        self.kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = [
-            (torch.zeros(num_blocks, n_kv, BLOCK_SIZE, cfg.head_dim,
-                         dtype=dtype, device=device),
-             torch.zeros(num_blocks, n_kv, BLOCK_SIZE, cfg.head_dim,
-                         dtype=dtype, device=device))
-            for _ in range(cfg.num_layers)
-        ]
+        self.specs = self.specs_for(model, cfg)
+        self.num_state_slots = num_state_slots
+        # one entry per layer, shaped by its spec (engine/cache_spec.py)
+        self.kv_caches: List = []
+        for spec in self.specs:
+            if isinstance(spec, PagedKV):
+                self.kv_caches.append(tuple(
+                    torch.zeros(num_blocks, spec.n_kv, BLOCK_SIZE,
+                                spec.head_dim, dtype=dtype, device=device)
+                    for _ in range(2)))
+            elif isinstance(spec, PagedLatent):
+                self.kv_caches.append(torch.zeros(
+                    num_blocks, BLOCK_SIZE, spec.width, dtype=dtype,
+                    device=device))
+            elif isinstance(spec, RecurrentState):
+                self.kv_caches.append(torch.zeros(
+                    max(num_state_slots, 1), spec.heads, spec.dim, spec.vdim,
+                    dtype=torch.float32, device=device))
+            elif isinstance(spec, SharedCache):
+                self.kv_caches.append(self.kv_caches[spec.source])
+            else:
+                raise TypeError(f"unknown cache spec {spec!r}")
         self.cpu_kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
+
+    @staticmethod
+    def specs_for(model, cfg: ModelConfig):
+        if hasattr(model, "cache_specs"):
+            return list(model.cache_specs())
+        n_kv = (model.local_kv_heads if hasattr(model, "local_kv_heads")
+                else cfg.num_kv_heads)
+        return default_specs(cfg, n_kv)
+
+    @property
+    def uses_state_slots(self) -> bool:
+        return needs_state_slots(self.specs)
+
+    def paged_tensors(self) -> List[torch.Tensor]:
+        """Every block-addressed cache tensor, each once (migration/export)."""
+        out = []
+        for spec, c in zip(self.specs, self.kv_caches):
+            if isinstance(spec, PagedKV):
+                out.extend(c)
+            elif isinstance(spec, PagedLatent):
+                out.append(c)
+        return out
 
     def alloc_cpu_caches(self, num_cpu_blocks: int):
         """Pinned host-DRAM tier for KV swapping."""
@@ -60,15 +98,21 @@ class ModelRunner:
                             n_kv_local: int,
                             gpu_memory_utilization: float = 0.85,
                             dtype_bytes: int = 2,
-                            max_blocks: Optional[int] = None) -> int:
-        """Size the block pool from actually-free HBM after weights load."""
+                            max_blocks: Optional[int] = None,
+                            specs=None, num_state_slots: int = 0) -> int:
+        """Size the block pool from actually-free HBM after weights load
+        (recurrent-state slots come off the budget first)."""
         if device.type == "cuda":
             free, _total = torch.cuda.mem_get_info(device)
             budget = int(free * gpu_memory_utilization)
         else:
             budget = 2 << 30  # CPU tests: 2 GiB worth of blocks
-        per_block = (2 * n_kv_local * BLOCK_SIZE * cfg.head_dim *
-                     dtype_bytes * cfg.num_layers)
+        if specs is None:
+            specs = default_specs(cfg, n_kv_local)
+        budget -= num_state_slots * sum(
+            s.slot_bytes() for s in specs if isinstance(s, RecurrentState))
+        per_block = max(sum(s.block_bytes(BLOCK_SIZE, dtype_bytes)
+                            for s in specs), 1)
         n = max(budget // per_block, 16)
         if max_blocks:
             n = min(n, max_blocks)
@@ -112,8 +156,13 @@ class ModelRunner:
         cu_q = [0]
         p_seq_lens: List[int] = []
         p_tables: List[List[int]] = []
+        p_ctx: List[int] = []
+        p_state: List[int] = []
+        d_state: List[int] = []
         for sp in plan.prefills:
             seq = sp.seq
+            p_ctx.append(sp.chunk_start)
+            p_state.append(seq.state_slot)
             chunk_toks = seq.prompt_token_ids[sp.chunk_start:
                                               sp.chunk_start + sp.chunk_len]
             if seq.mrope_pos is not None:
@@ -141,6 +190,7 @@ class ModelRunner:
             slots.append(bm.append_slot(seq))
             d_seq_lens.append(seq.total_len)
             d_tables.append(seq.block_table)
+            d_state.append(seq.state_slot)
 
         import numpy as _np
         if mrope_spans:
@@ -200,6 +250,13 @@ class ModelRunner:
                                           device=dev) if plan.decodes else None),
             decode_block_tables=pad_tables(d_tables) if plan.decodes else None,
         )
+        if self.uses_state_slots:
+            i32 = dict(dtype=torch.int32, device=dev)
+            if plan.prefills:
+                meta.prefill_ctx_lens = torch.tensor(p_ctx, **i32)
+                meta.prefill_state_slots = torch.tensor(p_state, **i32)
+            if plan.decodes:
+                meta.decode_state_slots = torch.tensor(d_state, **i32)
         input_ids = torch.tensor(tokens, dtype=torch.long, device=dev)
         pos_t = torch.from_numpy(pos_np).to(dev)
         return input_ids, pos_t, meta
@@ -317,6 +374,34 @@ class ModelRunner:
 
     prefill_graph = None
 
+    def _decode_graph_ok(self, plan: StepPlan) -> bool:
+        gr = self.graph_runner
+        return (gr is not None and not plan.prefills and bool(plan.decodes)
+                and gr.bucket_for(len(plan.decodes)) is not None
+                and all(s.total_len <= gr.max_blocks * BLOCK_SIZE
+                        for s in plan.decodes))
+
+    @torch.inference_mode()
+    def score(self, plan: StepPlan, bm, rows: List[int]) -> torch.Tensor:
+        """Run one step of the plan (same batch layout, caches and kernels
+        as execute) and return fp32 logits at the given batch rows instead
+        of sampling. Row r < num_prefill_tokens is a prefill-chunk token in
+        plan order; the decodes follow, one row each."""
+        if self._decode_graph_ok(plan):
+            logits = self._decode_graph_logits(plan, bm)
+            if not rows:
+                return logits.new_zeros((0, logits.shape[-1]),
+                                        dtype=torch.float32)
+            idx = torch.tensor(rows, dtype=torch.long, device=logits.device)
+            return logits[idx].float()
+        input_ids, positions, meta = self._build_batch(plan, bm)
+        self._tp_batch = None
+        hidden = self.model(input_ids, positions, self.kv_caches, meta)
+        if not rows:
+            return torch.zeros(0, self.cfg.vocab_size, dtype=torch.float32)
+        idx = torch.tensor(rows, dtype=torch.long, device=hidden.device)
+        return self.model.compute_logits(hidden[idx]).float()
+
     # ---- one step -----------------------------------------------------------
     @torch.inference_mode()
     def execute(self, plan: StepPlan, bm) -> Dict[str, int]:
@@ -333,11 +418,7 @@ class ModelRunner:
                 if (b is not None
                         and sp.chunk_start + b <= pg.max_model_len):
                     return self._execute_prefill_graph(sp, b)
-        gr = self.graph_runner
-        if (gr is not None and not plan.prefills and plan.decodes
-                and gr.bucket_for(len(plan.decodes)) is not None
-                and all(s.total_len <= gr.max_blocks * BLOCK_SIZE
-                        for s in plan.decodes)):
+        if self._decode_graph_ok(plan):
             return self._execute_decode_graph(plan, bm)
         input_ids, positions, meta = self._build_batch(plan, bm)
         tp_batch = getattr(self, "_tp_batch", None)
@@ -426,7 +507,9 @@ class ModelRunner:
         lps = self._logprobs(logits, [seq], toks)
         return {seq.request_id: (toks[0], lps.get(seq.request_id))}
 
-    def _execute_decode_graph(self, plan: StepPlan, bm) -> Dict[str, int]:
+    def _decode_graph_logits(self, plan: StepPlan, bm) -> torch.Tensor:
+        """Logits [n_decodes, vocab] of a decode-only plan via the captured
+        graph of its batch-size bucket."""
         import numpy as np
         seqs = plan.decodes
         n = len(seqs)
@@ -448,7 +531,14 @@ class ModelRunner:
             self._tp_bcast(dict(kind="graph", input_ids=input_ids,
                                 positions=positions, slots=slots,
                                 seq_lens=seq_lens, bt_rows=bt_rows))
-        logits = gr.run(input_ids, positions, slots, seq_lens, bt_rows)
+        state_slots = (np.asarray([s.state_slot for s in seqs], dtype=np.int32)
+                       if self.uses_state_slots else None)
+        return gr.run(input_ids, positions, slots, seq_lens, bt_rows,
+                      state_slots=state_slots)
+
+    def _execute_decode_graph(self, plan: StepPlan, bm) -> Dict[str, int]:
+        seqs = plan.decodes
+        logits = self._decode_graph_logits(plan, bm)
         tokens = self._sample(logits, seqs)
         lps = self._logprobs(logits, seqs, tokens)
         return {seq.request_id: (tok, lps.get(seq.request_id))

@@ -44,8 +44,10 @@ class EngineScheduler:
                  max_batched_tokens: int = 8192,
                  enable_chunked_prefill: bool = True,
                  prefill_hold_ms: float = 0.0,
-                 swap_out=None, swap_in=None):
+                 swap_out=None, swap_in=None, state_manager=None):
         self.bm = block_manager
+        # recurrent-state slot pool (None: the model keeps no such state)
+        self.sm = state_manager
         self.max_num_seqs = max_num_seqs
         self.max_batched_tokens = max_batched_tokens
         self.enable_chunked_prefill = enable_chunked_prefill
@@ -83,14 +85,14 @@ class EngineScheduler:
         for i, s in enumerate(self.running):
             if s.request_id == request_id:
                 s.status = SeqStatus.FINISHED_ABORT
-                self.bm.free(s)
+                self._release(s)
                 self.running.pop(i)
                 return s
         for i, s in enumerate(self.waiting):
             if s.request_id == request_id:
                 s.status = SeqStatus.FINISHED_ABORT
                 if s.block_table:
-                    self.bm.free(s)
+                    self._release(s)
                 del self.waiting[i]
                 return s
         for i, s in enumerate(self.swapped):
@@ -102,6 +104,12 @@ class EngineScheduler:
                 del self.swapped[i]
                 return s
         return None
+
+    def _release(self, seq: Sequence):
+        """Give back everything the sequence holds on the device."""
+        self.bm.free(seq)
+        if self.sm is not None:
+            self.sm.free(seq)
 
     # engine injects this (frees dram blocks of an aborted swapped seq)
     free_cpu_blocks = staticmethod(lambda seq: None)
@@ -130,7 +138,7 @@ class EngineScheduler:
                 self.swapped.append(victim)
                 self.num_swap_outs += 1
                 return
-        self.bm.free(victim)
+        self._release(victim)
         victim.status = SeqStatus.PREEMPTED
         victim.num_computed_tokens = 0
         n_out = len(victim.output_token_ids)
@@ -235,12 +243,16 @@ class EngineScheduler:
                 if not self.bm.can_allocate(seq, seq.prompt_len,
                                             reserve_blocks=reserved):
                     break
+                if self.sm is not None:
+                    if not self.sm.can_allocate():
+                        break
+                    self.sm.allocate(seq)
                 self.bm.allocate_prefill(seq)
             remaining = seq.prompt_len - seq.num_computed_tokens
             chunk = min(remaining, budget)
             if not self.enable_chunked_prefill and chunk < remaining:
                 if first_alloc:
-                    self.bm.free(seq)
+                    self._release(seq)
                     seq.num_computed_tokens = 0
                 break
             if chunk <= 0:
@@ -284,4 +296,6 @@ class EngineScheduler:
         for s in done:
             if not s.hold_blocks:
                 self.bm.free(s)
+            if self.sm is not None:
+                self.sm.free(s)
             self.running.remove(s)

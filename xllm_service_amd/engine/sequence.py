@@ -42,6 +42,7 @@ class Sequence:        # token lists element-wise (O(len) per membership test)
     block_table: List[int] = field(default_factory=list)
     cpu_block_table: List[int] = field(default_factory=list)  # dram tier
     num_computed_tokens: int = 0          # prompt tokens already prefilled
+    state_slot: int = -1                  # recurrent-state slot (-1 = none)
     preempt_count: int = 0
     # multimodal: pre-computed image embeddings substituted at placeholder
     # token positions during prefill (EPD E->P handoff)

@@ -1,13 +1,16 @@
 """Model configuration + named presets (random-init; no network access)."""
 from __future__ import annotations
 
+import json
+import os
 from dataclasses import dataclass, field
+from typing import List, Optional
 
 
 @dataclass
 class ModelConfig:
     name: str = "llama"
-    architecture: str = "llama"          # llama | opt | qwen2 | qwen2_vl
+    architecture: str = "llama"          # llama | opt | qwen2 | qwen2_vl | pugovik
     vocab_size: int = 128256
     hidden_size: int = 4096
     intermediate_size: int = 14336
@@ -103,7 +106,113 @@ PRESETS = {
 }
 
 
+@dataclass
+class HybridLayerConfig:
+    """One layer of a hybrid stack: which sequence mixer it has, the
+    mixer's sizes and constants, and its feed-forward (None = no FF)."""
+    type: str                      # latent_attention | lightning
+    mixer: dict = field(default_factory=dict)
+    mlp: Optional[dict] = None
+
+
+@dataclass
+class PugovikConfig(ModelConfig):
+    """Pugovik: per-layer choice of latent attention (a low-rank shared
+    key/value latent, optionally borrowed from an earlier layer) or decayed
+    linear attention with a recurrent state, routed-expert feed-forwards,
+    grouped RMS norms around every sublayer, gated + scaled residuals."""
+    layers: List[HybridLayerConfig] = field(default_factory=list)
+    norm_groups: int = 1
+    residual_mult: float = 1.0
+    model_dir: Optional[str] = None     # weights live here (None = random)
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return any(l.type == "lightning" for l in self.layers)
+
+
+def pugovik_from_dict(d: dict, name: str = "pugovik",
+                      model_dir: Optional[str] = None) -> PugovikConfig:
+    layers = [HybridLayerConfig(type=l["type"], mixer=dict(l["mixer"]),
+                                mlp=l.get("mlp"))
+              for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l.type not in ("latent_attention", "lightning"):
+            raise ValueError(f"layer {i}: unknown mixer type {l.type!r}")
+        src = l.mixer.get("kv_from")
+        if src is not None:
+            s = layers[src]
+            if (src >= i or s.type != "latent_attention"
+                    or "kv_from" in s.mixer):
+                raise ValueError(f"layer {i}: kv_from {src} is not an earlier "
+                                 "latent-attention layer with its own latent")
+    return PugovikConfig(
+        name=name, architecture="pugovik", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), num_layers=len(layers),
+        rms_eps=float(d["norm"]["eps"]),
+        norm_groups=int(d["norm"].get("groups", 1)),
+        residual_mult=float(d.get("residual_mult", 1.0)),
+        max_position=1 << 20, layers=layers, model_dir=model_dir)
+
+
+def load_model_dir(path: str) -> ModelConfig:
+    """Read <path>/config.json and pick the config class by its
+    `architecture` field."""
+    with open(os.path.join(path, "config.json")) as f:
+        d = json.load(f)
+    arch = str(d.get("architecture", "")).lower()
+    if arch == "pugovik":
+        return pugovik_from_dict(d, name=os.path.basename(
+            os.path.normpath(path)) or "pugovik", model_dir=path)
+    raise ValueError(f"{path}: unsupported architecture "
+                     f"{d.get('architecture')!r}")
+
+
+def _pugovik_preset(name, width, n_layers, heads, vocab=32000, experts=16,
+                    top=2, ff=None, every_attn=4, kv_rank=512, rot_dim=64):
+    """Synthetic Pugovik stacks for benchmarks: three decayed-linear layers
+    per latent-attention layer, the second attention layer of each pair
+    borrowing the first one's latent."""
+    hd = width // heads
+    layers, last_attn = [], None
+    for i in range(n_layers):
+        mlp = dict(kind="moe", expert=dict(ff=ff or width // 2),
+                   router=dict(experts=experts, top=top,
+                               groups=dict(count=4, keep=2)))
+        if i % every_attn == every_attn - 1:
+            mixer = dict(heads=heads, dim=hd, rot_dim=rot_dim, vdim=hd,
+                         kv_rank=kv_rank, scale=(hd + rot_dim) ** -0.5,
+                         rot=dict(base=10000.0, dims=rot_dim))
+            if last_attn is not None:
+                mixer["kv_from"] = last_attn
+                last_attn = None
+            else:
+                last_attn = i
+            layers.append(dict(type="latent_attention", mixer=mixer, mlp=mlp))
+        else:
+            decay = [1.0 - 2.0 ** -(2 + 6 * h / max(heads - 1, 1))
+                     for h in range(heads)]
+            layers.append(dict(type="lightning", mlp=mlp, mixer=dict(
+                heads=heads, dim=hd, vdim=hd, decay=decay)))
+    return pugovik_from_dict(dict(
+        architecture="Pugovik", vocab=vocab, width=width, layers=layers,
+        norm=dict(eps=1e-6, groups=4), residual_mult=0.5), name=name)
+
+
+PRESETS.update({
+    # CPU-test sized hybrid stack
+    "pugovik-tiny": _pugovik_preset("pugovik-tiny", 128, 4, 4, vocab=256,
+                                    experts=8, top=2, ff=64, every_attn=2,
+                                    kv_rank=48, rot_dim=16),
+    # bench stacks at the width of real deployments (random weights)
+    "pugovik-2k": _pugovik_preset("pugovik-2k", 2048, 8, 16),
+    "pugovik-4k": _pugovik_preset("pugovik-4k", 4096, 8, 32),
+})
+
+
 def get_config(name: str) -> ModelConfig:
+    if os.path.isdir(name):
+        return load_model_dir(name)
     if name not in PRESETS:
         raise KeyError(f"unknown model preset {name!r}; have {list(PRESETS)}")
     return PRESETS[name]

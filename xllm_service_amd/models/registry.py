@@ -18,4 +18,14 @@ def create_model(cfg: ModelConfig, dtype=torch.bfloat16):
         # (llama stack + qkv bias); the vision tower is a separate class
         from .qwen2_vl import Qwen2VLForCausalLM
         return Qwen2VLForCausalLM(cfg, dtype=dtype)
+    if cfg.architecture == "pugovik":
+        from .pugovik import PugovikForCausalLM
+        return PugovikForCausalLM(cfg, dtype=dtype)
     raise ValueError(f"unknown architecture {cfg.architecture}")
+
+
+def required_extensions(cfg: ModelConfig):
+    """In-tree HIP extension modules the model's GPU path loads."""
+    if cfg.architecture == "pugovik":
+        return ["_ops_hybrid"]
+    return ["_ops"]

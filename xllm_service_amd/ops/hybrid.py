@@ -1,0 +1,143 @@
+"""Hybrid-mixer ops: latent attention, decayed linear attention with a
+recurrent state, grouped RMS norms, gated residuals, routed experts.
+
+Same policy as the rest of `ops`: on a GPU the HIP extension (`_ops_hybrid`)
+is the only path and its absence raises; on CPU the fp32 torch references in
+`ops.ref` run. Activations may be bf16 or fp32; norms, scores, softmax
+weights, recurrent state, router and residual are fp32 in both.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import ref
+
+_ext = None
+
+
+def _hyb():
+    global _ext
+    if _ext is None:
+        try:
+            from xllm_service_amd import _ops_hybrid as m
+        except ImportError as e:
+            raise RuntimeError(
+                "xllm_service_amd._ops_hybrid (gfx950 HIP extension) is not "
+                "built but a GPU op was requested. Build it with: "
+                "XLLM_BUILD_EXT=_ops_hybrid python setup.py build_ext "
+                "--inplace") from e
+        _ext = m
+    return _ext
+
+
+def group_rmsnorm(x, w, eps: float, groups: int, out_dtype=None):
+    out_dtype = out_dtype or x.dtype
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _hyb().group_rmsnorm(out, x, w, eps, groups)
+        return out
+    return ref.group_rmsnorm(x, w, eps, groups, out_dtype)
+
+
+def gated_norm_residual(res, y, gate, gate_bias, w, ls, mult: float,
+                        eps: float, groups: int):
+    """res (fp32, in place) += mult * ls * group_rmsnorm(y * sigmoid(gate +
+    gate_bias)) * w."""
+    if res.is_cuda:
+        _hyb().gated_norm_residual(res, y, gate, gate_bias, w, ls, mult, eps,
+                                   groups)
+        return res
+    return ref.gated_norm_residual(res, y, gate, gate_bias, w, ls, mult, eps,
+                                   groups)
+
+
+def norm_sigmoid_gate(o, w: Optional[torch.Tensor], gate, eps: float,
+                      out_dtype):
+    """(rmsnorm(o) * w if w is given else o) * sigmoid(gate); o fp32 2-D."""
+    if o.is_cuda:
+        out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+        _hyb().norm_sigmoid_gate(out, o, w, gate, eps)
+        return out
+    return ref.norm_sigmoid_gate(o, w, gate, eps, out_dtype)
+
+
+def silu_mul(x):
+    if x.is_cuda:
+        out = torch.empty(x.shape[:-1] + (x.shape[-1] // 2,), dtype=x.dtype,
+                          device=x.device)
+        _hyb().silu_mul(out, x)
+        return out
+    return ref.silu_mul(x)
+
+
+def rope_interleaved_(x, positions, inv_freq, mscale: float, off: int,
+                      rot_dims: int):
+    """Rotate x[..., off:off+rot_dims] ([T, H, D] view) in place."""
+    if x.is_cuda:
+        _hyb().rope_interleaved(x, positions, inv_freq, mscale, off, rot_dims)
+        return x
+    x[..., off:off + rot_dims] = ref.rope_interleaved(
+        x[..., off:off + rot_dims], positions, inv_freq, mscale, rot_dims)
+    return x
+
+
+def latent_kv_store(dkv, norm_w, eps, positions, inv_freq, mscale, rot_dims,
+                    cache, slot_mapping, kv_rank):
+    if dkv.is_cuda:
+        _hyb().latent_kv_store(cache, dkv, norm_w, eps, positions, inv_freq,
+                               mscale, rot_dims, slot_mapping, kv_rank)
+        return
+    ref.latent_kv_store(dkv, norm_w, eps, positions, inv_freq, mscale,
+                        rot_dims, cache, slot_mapping, kv_rank)
+
+
+def latent_attn(q, cache, block_tables, cu_q, seq_lens, scale, kv_rank, out):
+    """out fp32 [T, H, kv_rank] (written). cu_q None: decode rows."""
+    if q.is_cuda:
+        _hyb().latent_attn(out, q, cache, block_tables, cu_q, seq_lens, scale,
+                           kv_rank)
+        return out
+    if cu_q is None:
+        cu_q = torch.arange(q.shape[0] + 1, dtype=torch.int32)
+    out.copy_(ref.latent_attn(q, cache, block_tables, cu_q, seq_lens, scale,
+                              kv_rank))
+    return out
+
+
+def decay_attn(q, k, v, decay, state, slots, cu_q, ctx_lens, out):
+    """out fp32 [T, H, Dv] (written); q/k/v are pre-activation row views
+    [T, H*D] / [T, H*Dv]; state fp32 [slots, H, D, Dv] updated in place."""
+    if q.is_cuda:
+        _hyb().decay_attn(out, q, k, v, decay, state, slots, cu_q, ctx_lens)
+        return out
+    H, D, Dv = state.shape[1:]
+    T = q.shape[0]
+    if cu_q is None:
+        cu_q = torch.arange(T + 1, dtype=torch.int32)
+    out.copy_(ref.decay_linear_attn(
+        q.reshape(T, H, D), k.reshape(T, H, D), v.reshape(T, H, Dv), decay,
+        state, slots, cu_q, ctx_lens))
+    return out
+
+
+def moe_route(h, w_router, top: int, n_groups: int, keep: int):
+    if h.is_cuda:
+        T = h.shape[0]
+        ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
+        wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
+        _hyb().moe_route(ids, wts, h, w_router, top, n_groups, keep)
+        return ids, wts
+    return ref.moe_route(h, w_router, top, n_groups, keep)
+
+
+def moe_combine(y, rows, wts, tokens: int):
+    """fp32 [tokens, width] = sum_k wts[t, k] * y[rows[t, k]]."""
+    width = y.shape[-1]
+    if y.is_cuda:
+        out = torch.empty(tokens, width, dtype=torch.float32, device=y.device)
+        _hyb().moe_combine(out, y.view(-1, width), rows, wts)
+        return out
+    yy = y.reshape(-1, width).float()[rows.long()]          # [T, top, W]
+    return (yy * wts[:, :, None]).sum(1)
