@@ -22,6 +22,23 @@ log = logging.getLogger("xllm.graph")
 BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
 
 
+def _wait_staging(pin: dict) -> None:
+    """Block until the async host-to-device copies of the previous replay
+    have read the pinned staging buffers; only then may the host refill
+    them. A caller that syncs every step (sampling does) never waits here,
+    one that replays without reading results back would otherwise race."""
+    ev = pin.get("copied")
+    if ev is not None:
+        ev.synchronize()
+
+
+def _mark_staging(pin: dict) -> None:
+    ev = pin.get("copied")
+    if ev is None:
+        ev = pin["copied"] = torch.cuda.Event()
+    ev.record()
+
+
 class DecodeGraphRunner:
     def __init__(self, model, kv_caches, device, max_model_len: int = 4096,
                  max_batch: int = 256):
@@ -128,6 +145,7 @@ class DecodeGraphRunner:
         bs = self.bucket_for(n)
         graph, static, logits = self.graphs[bs]
         pin = self._pinned[bs]
+        _wait_staging(pin)
         i64 = pin["i64"].numpy()
         i64[0, :n] = input_ids
         i64[1, :n] = positions
@@ -150,6 +168,7 @@ class DecodeGraphRunner:
         static["seq_lens"].copy_(pin["seq_lens"], non_blocking=True)
         static["block_tables"][:n].copy_(pin["block_tables"][:n],
                                          non_blocking=True)
+        _mark_staging(pin)
         graph.replay()
         return logits[:n]
 
@@ -256,6 +275,7 @@ class PrefillGraphRunner:
         L = len(tokens)
         graph, static, hidden = self.graphs[B]
         pin = self._pinned[B]
+        _wait_staging(pin)
         i64 = pin["i64"].numpy()
         i64[0, :L] = tokens
         i64[1, :L] = positions
@@ -271,5 +291,6 @@ class PrefillGraphRunner:
         static["slot_mapping"].copy_(pin["i64"][2], non_blocking=True)
         static["seq_lens"].copy_(pin["seq_len"], non_blocking=True)
         static["block_tables"].copy_(pin["block_tables"], non_blocking=True)
+        _mark_staging(pin)
         graph.replay()
         return hidden
