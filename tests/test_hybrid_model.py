@@ -130,9 +130,14 @@ def test_layers_residual_stream(root, target, name):
     trail = o_forward(cfg, w, toks)[1]
     assert len(seen) == len(trail)
     for i, (a, b) in enumerate(zip(seen, trail)):
-        tol = 2e-4 if target[1] == torch.float32 else 0.08
-        err = float((a.double() - b).abs().max() / b.abs().max())
-        assert err < tol, (name, i, err)
+        # per token; in bf16 a router near-tie may flip and move that token
+        # from there on (the fp32 run above is the strict one)
+        err = ((a.double() - b).norm(dim=-1) / b.norm(dim=-1))
+        if target[1] == torch.float32:
+            assert float(err.max()) < 2e-4, (name, i, float(err.max()))
+        else:
+            assert float(err.median()) < 0.05, (name, i, err)
+            assert float((err > 0.15).float().mean()) <= 0.25, (name, i, err)
 
 
 @pytest.mark.parametrize("target", TARGETS)
