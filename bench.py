@@ -59,8 +59,13 @@ def parse_args():
                     help="serving: timed completed requests; "
                          "engine: timed engine steps")
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--mode", choices=("serving", "engine"),
-                    default="serving")
+    ap.add_argument("--mode", choices=("serving", "engine", "hybrid"),
+                    default="serving",
+                    help="hybrid: prefill/decode throughput and per-kernel "
+                         "rates of the pugovik stacks beside equal-size "
+                         "llama stacks (one GPU; prints one JSON line per "
+                         "measurement, not the headline record)")
+    ap.add_argument("--hybrid-sizes", default="2k,4k")
     ap.add_argument("--model", default="llama-3-8b")
     ap.add_argument("--concurrency", type=int, default=128,
                     help="ramp/calibration concurrency per decode GPU "
@@ -87,6 +92,172 @@ def parse_args():
     ap.add_argument("--max-kv-blocks", type=int, default=0)
     ap.add_argument("--startup-timeout", type=float, default=900.0)
     return ap.parse_args()
+
+
+# --------------------------------------------------------------------------
+# hybrid mode: pugovik-<size> beside llama-<size>, end to end and per kernel
+# --------------------------------------------------------------------------
+def _time_gpu(fn, iters=10, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(
+        enable_timing=True)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters * 1e-3
+
+
+def _hybrid_end_to_end(name, device, prompt_len, batch, ctx, steps):
+    """(prefill tok/s for one prompt_len prompt, decode tok/s at `batch`
+    sequences of ~ctx tokens through the captured decode graph)."""
+    from xllm_service_amd.engine.engine import LLMEngine
+    from xllm_service_amd.engine.sampling import SamplingParams
+    from xllm_service_amd.models.config import get_config
+    cfg = get_config(name)
+    blocks = (batch * (ctx + steps + 64) + prompt_len) // 16 + 64
+    eng = LLMEngine(name, device=device, max_num_seqs=batch,
+                    max_batched_tokens=max(prompt_len, 8192),
+                    max_kv_blocks=blocks, max_model_len=max(prompt_len, ctx)
+                    + steps + 128, state_slots=batch + 1, seed=0,
+                    enable_prefix_caching=False, swap_space_mb=0)
+    g = torch.Generator().manual_seed(0)
+    mk = lambda n: torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist()
+    one = SamplingParams(max_tokens=1, ignore_eos=True)
+    eng.generate([mk(prompt_len)], one)                       # warm
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        eng.generate([mk(prompt_len)], one)
+    torch.cuda.synchronize()
+    prefill = reps * prompt_len / (time.perf_counter() - t0)
+    for i in range(batch):
+        eng.add_request(f"d{i}", mk(ctx), SamplingParams(
+            max_tokens=steps + 16, ignore_eos=True))
+    while any(not s.prefill_done for s in eng.seqs.values()):
+        eng.step()
+    for _ in range(8):
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n = 0
+    for _ in range(steps):
+        n += sum(len(o.new_token_ids) for o in eng.step())
+    torch.cuda.synchronize()
+    decode = n / (time.perf_counter() - t0)
+    del eng
+    torch.cuda.empty_cache()
+    return prefill, decode
+
+
+def _hybrid_kernels(size, device, T, batch, ctx):
+    """Achieved rates of the mixer kernels at one layer's shapes: bytes that
+    must move (GB/s) for the decode kernels, useful FLOP/s for prefill."""
+    from xllm_service_amd import ops
+    from xllm_service_amd.models.config import get_config
+    from xllm_service_amd.ops import hybrid as hops
+    pc, lc = get_config(f"pugovik-{size}"), get_config(f"llama-{size}")
+    lat = next(l.mixer for l in pc.layers if l.type == "latent_attention")
+    lin = next(l.mixer for l in pc.layers if l.type == "lightning")
+    bf = dict(dtype=torch.bfloat16, device=device)
+    i32 = dict(dtype=torch.int32, device=device)
+    out = []
+    nblk = (max(T, ctx) + 15) // 16
+    # ---- latent attention vs paged attention -----------------------------
+    H, r, rd = lat["heads"], lat["kv_rank"], lat["rot_dim"]
+    W = r + rd
+    cache = torch.randn(batch * nblk, 16, W, **bf)
+    tab = torch.arange(batch * nblk, **i32).view(batch, nblk)
+    q = torch.randn(T, H, W, **bf)
+    o = torch.empty(T, H, r, dtype=torch.float32, device=device)
+    cu = torch.tensor([0, T], **i32)
+    sl = torch.tensor([T], **i32)
+    t = _time_gpu(lambda: hops.latent_attn(q, cache, tab[:1], cu, sl, 0.1, r,
+                                           o), 3, 1)
+    fl = 2.0 * H * (W + r) * T * (T + 1) / 2
+    out.append(("latent_attn prefill", t, fl / t / 1e12, "TFLOP/s"))
+    qd = torch.randn(batch, H, W, **bf)
+    od = torch.empty(batch, H, r, dtype=torch.float32, device=device)
+    sld = torch.full((batch,), ctx, **i32)
+    t = _time_gpu(lambda: hops.latent_attn(qd, cache, tab, None, sld, 0.1, r,
+                                           od))
+    out.append(("latent_attn decode", t, batch * ctx * W * 2 / t / 1e9,
+                "GB/s"))
+    Hq, Hk, D = lc.num_heads, lc.num_kv_heads, lc.head_dim
+    kc = torch.randn(batch * nblk, Hk, 16, D, **bf)
+    vc = torch.randn(batch * nblk, Hk, 16, D, **bf)
+    ql = torch.randn(T, Hq, D, **bf)
+    if D == 128:
+        t = _time_gpu(lambda: ops.paged_attn_prefill(ql, kc, vc, tab[:1], cu,
+                                                     sl, 0.1), 3, 1)
+        out.append(("paged_attn prefill (llama)", t,
+                    4.0 * Hq * D * T * (T + 1) / 2 / t / 1e12, "TFLOP/s"))
+    qld = torch.randn(batch, Hq, D, **bf)
+    t = _time_gpu(lambda: ops.paged_attn_decode(qld, kc, vc, tab, sld, 0.1))
+    out.append(("paged_attn decode (llama)", t,
+                batch * ctx * Hk * D * 2 * 2 / t / 1e9, "GB/s"))
+    # ---- decayed linear attention ----------------------------------------
+    Hh, Dk, Dv = lin["heads"], lin["dim"], lin["vdim"]
+    dec = torch.tensor(lin["decay"], dtype=torch.float32, device=device)
+    st = torch.zeros(batch, Hh, Dk, Dv, dtype=torch.float32, device=device)
+    qkv = torch.randn(T, 2 * Hh * Dk + Hh * Dv, **bf)
+    oo = torch.empty(T, Hh, Dv, dtype=torch.float32, device=device)
+    t = _time_gpu(lambda: hops.decay_attn(
+        qkv[:, :Hh * Dk], qkv[:, Hh * Dk:2 * Hh * Dk], qkv[:, 2 * Hh * Dk:],
+        dec, st, torch.zeros(1, **i32), cu, torch.zeros(1, **i32), oo), 3, 1)
+    out.append(("decay_attn prefill", t, 4.0 * Hh * Dk * Dv * T / t / 1e12,
+                "TFLOP/s (recurrence form)"))
+    qkvd = torch.randn(batch, 2 * Hh * Dk + Hh * Dv, **bf)
+    ood = torch.empty(batch, Hh, Dv, dtype=torch.float32, device=device)
+    sls = torch.arange(batch, **i32)
+    cx = torch.full((batch,), ctx, **i32)
+    t = _time_gpu(lambda: hops.decay_attn(
+        qkvd[:, :Hh * Dk], qkvd[:, Hh * Dk:2 * Hh * Dk], qkvd[:, 2 * Hh * Dk:],
+        dec, st, sls, None, cx, ood))
+    out.append(("decay_attn decode", t,
+                batch * Hh * Dk * Dv * 4 * 2 / t / 1e9, "GB/s"))
+    # ---- norms -------------------------------------------------------------
+    Wd = pc.hidden_size
+    x = torch.randn(T, Wd, dtype=torch.float32, device=device)
+    w = torch.ones(Wd, dtype=torch.float32, device=device)
+    t = _time_gpu(lambda: hops.group_rmsnorm(x, w, 1e-6, pc.norm_groups,
+                                             torch.bfloat16))
+    out.append(("group_rmsnorm fp32->bf16", t, T * Wd * 6 / t / 1e9, "GB/s"))
+    y = torch.randn(T, Wd, **bf)
+    gt = torch.randn(T, Wd, **bf)
+    t = _time_gpu(lambda: hops.gated_norm_residual(x, y, gt, w, w, w, 0.5,
+                                                   1e-6, pc.norm_groups))
+    out.append(("gated_norm_residual", t, T * Wd * 12 / t / 1e9, "GB/s"))
+    xb, rb, wb = torch.randn(T, Wd, **bf), torch.randn(T, Wd, **bf), \
+        torch.ones(Wd, **bf)
+    t = _time_gpu(lambda: ops.fused_add_rmsnorm(xb, rb, wb, 1e-6))
+    out.append(("fused_add_rmsnorm (llama)", t, T * Wd * 8 / t / 1e9, "GB/s"))
+    return out
+
+
+def run_hybrid_mode(args, device):
+    assert torch.cuda.is_available(), "hybrid mode measures the HIP path"
+    for size in args.hybrid_sizes.split(","):
+        T, batch, ctx = 4096, 32, 2048
+        for name, t, rate, unit in _hybrid_kernels(size, device, T, batch,
+                                                   ctx):
+            print(json.dumps(dict(kind="kernel", size=size, kernel=name,
+                                  ms=round(t * 1e3, 4), rate=round(rate, 2),
+                                  unit=unit, tokens=T, batch=batch, ctx=ctx)),
+                  flush=True)
+        for fam in ("pugovik", "llama"):
+            pre, dec = _hybrid_end_to_end(f"{fam}-{size}", device, T, batch,
+                                          1024, args.steps)
+            print(json.dumps(dict(kind="end_to_end", model=f"{fam}-{size}",
+                                  prefill_tok_s=round(pre, 1),
+                                  prefill_len=T,
+                                  decode_tok_s=round(dec, 1), batch=batch,
+                                  ctx=1024, dtype="bf16",
+                                  data="synthetic")), flush=True)
 
 
 # --------------------------------------------------------------------------
@@ -712,7 +883,9 @@ def main():
         nd = sum(1 for x in r if x != "PREFILL") or 1
         args.push_interval_ms = 25.0 * max(1.0, nd / 2.0)
 
-    if args.mode == "engine":
+    if args.mode == "hybrid":
+        run_hybrid_mode(args, args.device or f"cuda:{local_rank}")
+    elif args.mode == "engine":
         device = args.device or (f"cuda:{local_rank}" if use_gpu else "cpu")
         run_engine_mode(args, rank, world, local_rank, use_gpu, dist,
                         device, model_name)

@@ -53,7 +53,7 @@ ext_modules = [
         sources=[
             os.path.join(HYB, f)
             for f in ("bindings.cpp", "norms.hip", "latent_attn.hip",
-                      "decay_attn.hip", "moe.hip")
+                      "latent_attn_mfma.hip", "decay_attn.hip", "moe.hip")
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],

@@ -182,7 +182,7 @@ def lin_layer(heads=3, dim=8, vdim=12, decay=None, mlp=None):
                 mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=decay))
 
 
-def lat_layer(heads=2, dim=12, rot_dim=8, vdim=10, kv_rank=20, dims=None,
+def lat_layer(heads=2, dim=12, rot_dim=8, vdim=10, kv_rank=24, dims=None,
               scaling=True, kv_from=None, mlp=None, base=10000.0):
     rot = dict(base=base, dims=dims or rot_dim)
     if scaling:

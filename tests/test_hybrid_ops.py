@@ -161,7 +161,9 @@ def test_latent_attn_standout_keys(dev, dt):
 
 @pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("heads,r,rd", [(1, 5, 2), (5, 70, 6), (4, 130, 0)])
+@pytest.mark.parametrize("heads,r,rd", [(1, 5, 2), (5, 70, 6), (4, 130, 0),
+                                        (5, 80, 16), (3, 200, 24),
+                                        (17, 512, 64), (40, 48, 8)])
 def test_latent_attn_batch_of_unequal_sequences(dev, dt, heads, r, rd):
     if dev == "cpu" and dt != torch.float32:
         pytest.skip("cpu path is fp32")
@@ -346,3 +348,30 @@ def test_norm_sigmoid_gate(dev):
     got = H.norm_sigmoid_gate(o.to(dev), None, gate.to(dev), 1e-5,
                               torch.float32)
     _close(got, o.to(F64) * torch.sigmoid(gate.to(F64)), 3e-6)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("heads,r,rd", [(2, 40, 8), (19, 128, 32)])
+def test_latent_attn_decode_rows_of_unequal_context(dev, dt, heads, r, rd):
+    """Decode rows whose contexts differ widely (the kernel may split long
+    contexts over several workgroups and merge the parts)."""
+    if dev == "cpu" and dt != torch.float32:
+        pytest.skip("cpu path is fp32")
+    bs, W = 16, r + rd
+    g = torch.Generator().manual_seed(13)
+    lens = [1, 700, 33, 64, 65, 257]
+    nb = (max(lens) + bs - 1) // bs
+    tables = _scrambled_tables(len(lens), nb, len(lens) * nb + 3, 14)
+    cache = (torch.randn(len(lens) * nb + 3, bs, W, generator=g) * 0.5).to(dt)
+    q = torch.randn(len(lens), heads, W, generator=g).to(dt)
+    out = torch.empty(len(lens), heads, r, dtype=torch.float32, device=dev)
+    H.latent_attn(q.to(dev), cache.to(dev), tables.to(dev), None,
+                  torch.tensor(lens, dtype=torch.int32, device=dev), 0.2, r,
+                  out)
+    for s, L in enumerate(lens):
+        rows = torch.stack([cache[int(tables[s, p // bs]), p % bs]
+                            for p in range(L)])
+        for h in range(heads):
+            _close(out[s, h], _plain_latent_attn(q[s, h], rows, 0.2, r, L),
+                   _tol(dt))

@@ -6,6 +6,8 @@
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
 
+#include <algorithm>
+
 namespace xllm {
 namespace hyb {
 template <typename TI, typename TO>
@@ -31,6 +33,11 @@ template <typename T>
 void launch_latent_attn(float*, const T*, const T*, const int*, const int*,
                         const int*, int, int, int, int, int, int, int, float,
                         long, hipStream_t);
+int latent_attn_mfma_class(int W, int r);
+void launch_latent_attn_mfma(float*, float*, float*, const unsigned short*,
+                             const unsigned short*, const int*, const int*,
+                             const int*, int, int, int, int, int, int, int,
+                             float, int, hipStream_t);
 template <typename T>
 void launch_decay_attn(float*, const T*, const T*, const T*, const float*,
                        float*, const int*, const int*, const int*, int, int,
@@ -210,6 +217,29 @@ void latent_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables,
     cu = ptr<int>(*cu_q);
   } else {
     TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  // bf16: MFMA kernel when the sizes fit one of its instantiations
+  if (is_bf16(q) && hy::latent_attn_mfma_class(W, r) != 0) {
+    int n_part = 1;
+    Tensor ws_acc, ws_ml;
+    if (cu == nullptr) {
+      // decode: split the context over workgroups when tokens alone do not
+      // fill the chip (sizes known on the host only: no sync)
+      const int tps = (H + 63) / 64;
+      const long max_tiles = ((long)block_tables.size(1) * cache.size(1) + 31) / 32;
+      n_part = (int)std::min<long>(std::min<long>(16, max_tiles),
+                                   std::max<long>(1, 512 / ((long)T * tps)));
+    }
+    if (n_part > 1) {
+      ws_acc = torch::empty({(long)T * H * n_part, (long)r}, out.options());
+      ws_ml = torch::empty({(long)T * H * n_part, 2}, out.options());
+    }
+    hy::launch_latent_attn_mfma(
+        ptr<float>(out), n_part > 1 ? ptr<float>(ws_acc) : nullptr,
+        n_part > 1 ? ptr<float>(ws_ml) : nullptr, ptr<bf>(q), ptr<bf>(cache),
+        ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, H, r,
+        W - r, cache.size(1), block_tables.size(1), scale, n_part, cur());
+    return;
   }
   const int nw = H < 4 ? H : 4;
   TORCH_CHECK((size_t)nw * W * 4 <= 64 * 1024, "query row too wide for LDS");

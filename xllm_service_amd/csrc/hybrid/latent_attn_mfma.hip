@@ -1,0 +1,290 @@
+// MFMA latent attention (bf16 activations/cache) for gfx950.
+//
+// All heads of a token attend to the SAME cached rows [latent | rotated key],
+// so (query, head) pairs are just rows of one big query matrix: row
+// rho = query * H + head of a sequence's chunk, contiguous in the [T, H, W]
+// query tensor. A workgroup (4 waves) owns 64 such rows, a wave 16.
+//
+// Per 32-key tile:
+//   S^T[key][row] = K[key][:] . Q[row][:]      A = K rows, 16 B per lane straight
+//                                              from the paged cache; B = Q, held
+//                                              in registers for the whole kernel
+//   online softmax per row in fp32 (a lane holds 8 keys of ONE row)
+//   O^T[col][row] += V^T[col][key] P^T[key][row]
+//                                              A = V^T from LDS (the tile is
+//                                              staged transposed once per
+//                                              workgroup), B = the lane's own 8
+//                                              weights: no exchange needed
+// The C layout of S^T hands each lane keys g*4+r of both 16-key halves; the
+// staged V^T stores key columns in exactly that order, so P never moves.
+// Softmax weights stay 32-bit: p is split exactly into three bf16 terms
+// (8+8+8 mantissa bits) and each term gets its own MFMA into the fp32
+// accumulator.
+//
+// Decode splits the context over `n_part` workgroups per token; partial
+// (acc, max, sum) triples are merged by a second small kernel.
+//
+// Fragment layouts of __builtin_amdgcn_mfma_f32_16x16x32_bf16 (lane l):
+//   A[l&15][(l>>4)*8 + j], B[(l>>4)*8 + j][l&15], C[(l>>4)*4 + r][l&15].
+#include "hybrid_common.h"
+
+namespace xllm {
+namespace hyb {
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+constexpr int LM_ROWS = 64;     // rows per workgroup
+constexpr int LM_KT = 32;       // keys per tile
+constexpr int LM_VS = 40;       // V^T row stride in LDS (32 keys + pad)
+
+struct alignas(16) u16x8 { unsigned short x[8]; };
+
+XLLM_DEV bf16x8 ld8(const unsigned short* p) {
+  return *reinterpret_cast<const bf16x8*>(p);
+}
+
+template <int KQ, int NO>
+__global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
+    float* __restrict__ out, float* __restrict__ ws_acc,
+    float* __restrict__ ws_ml, const unsigned short* __restrict__ q,
+    const unsigned short* __restrict__ cache,
+    const int* __restrict__ block_tables, const int* __restrict__ cu_q,
+    const int* __restrict__ seq_lens, int n_seqs, int heads, int r, int rd,
+    int block_size, int table_width, float scale, int n_part) {
+  extern __shared__ unsigned short vt[];          // [rp][LM_VS]
+  const int W = r + rd;
+  const int Wp = (W + 31) & ~31;
+  const int rp = (r + 15) & ~15;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int g = lane >> 4, n = lane & 15;
+
+  // ---- which sequence / row tile is this workgroup ----------------------
+  int s, lt, qlen, q0;
+  const int bid = blockIdx.x;
+  if (cu_q == nullptr) {
+    const int tps = (heads + LM_ROWS - 1) / LM_ROWS;
+    s = bid / tps; lt = bid - s * tps; qlen = 1; q0 = s;
+    if (s >= n_seqs) return;
+  } else {
+    int acc = 0; s = -1; lt = 0;
+    for (int i = 0; i < n_seqs; ++i) {
+      const int nt = ((cu_q[i + 1] - cu_q[i]) * heads + LM_ROWS - 1) / LM_ROWS;
+      if (bid < acc + nt) { s = i; lt = bid - acc; break; }
+      acc += nt;
+    }
+    if (s < 0) return;
+    q0 = cu_q[s]; qlen = cu_q[s + 1] - q0;
+  }
+  const int rows_in_seq = qlen * heads;
+  const int ctx = seq_lens[s] - qlen;
+  const int row0 = lt * LM_ROWS;
+  const int last_row = min(row0 + LM_ROWS, rows_in_seq) - 1;
+  const int kmax = ctx + last_row / heads + 1;       // keys any row here sees
+  const int n_tiles = (kmax + LM_KT - 1) / LM_KT;
+  const int tpp = (n_tiles + n_part - 1) / n_part;
+  const int t_begin = blockIdx.y * tpp;
+  const int t_end = min(n_tiles, t_begin + tpp);
+  const int* table = block_tables + (long)s * table_width;
+
+  // ---- this lane's row -----------------------------------------------------
+  const int rho = row0 + wv * 16 + n;
+  const bool wave_on = row0 + wv * 16 < rows_in_seq;
+  const bool row_ok = rho < rows_in_seq;
+  const int limit = row_ok ? ctx + rho / heads + 1 : 0;
+  const long grow = (long)q0 * heads + rho;          // row in [T*H]
+
+  bf16x8 qf[KQ];
+#pragma unroll
+  for (int kc = 0; kc < KQ; ++kc) {
+    const int col = kc * 32 + g * 8;
+    bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+    qf[kc] = (row_ok && col < W) ? ld8(q + grow * W + col) : z;
+  }
+  f32x4 acc[NO];
+#pragma unroll
+  for (int i = 0; i < NO; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  const int CH = rp >> 3;                            // 16 B chunks per row
+  for (int t = t_begin; t < t_end; ++t) {
+    const int k0 = t * LM_KT;
+    __syncthreads();
+    // stage V^T (first rp columns of each cached row), keys permuted so
+    // that position g*8 + j holds key g*4 + j (j<4) / 16 + g*4 + j-4
+    for (int c = tid; c < LM_KT * CH; c += 256) {
+      const int kl = c / CH, part = c - kl * CH;
+      const int key = k0 + kl, col = part * 8;
+      u16x8 v8 = {{0, 0, 0, 0, 0, 0, 0, 0}};
+      if (key < kmax && col < W) {
+        const long blk = table[key / block_size];
+        v8 = *reinterpret_cast<const u16x8*>(
+            cache + (blk * block_size + key % block_size) * (long)W + col);
+      }
+      const int half = kl >> 4, k16 = kl & 15;
+      const int pos = (k16 >> 2) * 8 + half * 4 + (k16 & 3);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(col + e) * LM_VS + pos] = v8.x[e];
+    }
+    __syncthreads();
+    if (!wave_on) continue;
+    // ---- scores ------------------------------------------------------------
+    float sc[8];
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int key = k0 + h2 * 16 + n;              // A row of this lane
+      const bool kok = key < kmax;
+      const unsigned short* krow = cache;
+      if (kok) {
+        const long blk = table[key / block_size];
+        krow = cache + (blk * block_size + key % block_size) * (long)W;
+      }
+      f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < KQ; ++kc) {
+        if (kc * 32 < Wp) {
+          const int col = kc * 32 + g * 8;
+          bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+          const bf16x8 a = (kok && col < W) ? ld8(krow + col) : z;
+          sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kc], sacc, 0, 0,
+                                                         0);
+        }
+      }
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int kk = k0 + h2 * 16 + g * 4 + rr;    // C row = key
+        sc[h2 * 4 + rr] = (kk < limit) ? sacc[rr] * scale : -INFINITY;
+      }
+    }
+    float mloc = sc[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mloc = fmaxf(mloc, sc[i]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float m_new = fmaxf(m, mloc);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __expf(m - m_use);
+    float p[8], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { p[i] = __expf(sc[i] - m_use); psum += p[i]; }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    // exact 3-way bf16 split of the fp32 weights
+    bf16x8 b1, b2, b3;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const unsigned short h1 = f32_to_bf16(p[i]);
+      const float r1 = p[i] - bf16_to_f32(h1);
+      const unsigned short h2 = f32_to_bf16(r1);
+      const float r2 = r1 - bf16_to_f32(h2);
+      b1[i] = (short)h1; b2[i] = (short)h2; b3[i] = (short)f32_to_bf16(r2);
+    }
+#pragma unroll
+    for (int no = 0; no < NO; ++no) {
+      if (no * 16 < rp) {
+        acc[no] *= alpha;
+        const bf16x8 a = ld8(vt + (no * 16 + n) * LM_VS + g * 8);
+        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, acc[no], 0, 0, 0);
+        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, acc[no], 0, 0, 0);
+        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b3, acc[no], 0, 0, 0);
+      }
+    }
+  }
+  if (!wave_on || !row_ok) return;
+  // acc[no][rr] = O^T[col = no*16 + g*4 + rr][row n]
+  if (n_part == 1) {
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    float* orow = out + grow * r;
+#pragma unroll
+    for (int no = 0; no < NO; ++no)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int col = no * 16 + g * 4 + rr;
+        if (no * 16 < rp && col < r) orow[col] = acc[no][rr] * inv;
+      }
+  } else {
+    // partials are indexed by the OUTPUT row: [row][part]
+    const long base = grow * n_part + blockIdx.y;
+    float* arow = ws_acc + base * r;
+#pragma unroll
+    for (int no = 0; no < NO; ++no)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int col = no * 16 + g * 4 + rr;
+        if (no * 16 < rp && col < r) arow[col] = acc[no][rr];
+      }
+    if (g == 0) { ws_ml[base * 2] = m; ws_ml[base * 2 + 1] = l; }
+  }
+}
+
+// out[row] = sum_p acc[row][p] e^(m_p - M) / sum_p l_p e^(m_p - M)
+__global__ void latent_attn_merge_kernel(float* __restrict__ out,
+                                         const float* __restrict__ ws_acc,
+                                         const float* __restrict__ ws_ml,
+                                         int r, int n_part) {
+  const long row = blockIdx.x;
+  float M = -INFINITY;
+  for (int p = 0; p < n_part; ++p)
+    M = fmaxf(M, ws_ml[(row * n_part + p) * 2]);
+  if (M == -INFINITY) M = 0.f;
+  float L = 0.f;
+  for (int p = 0; p < n_part; ++p)
+    L += ws_ml[(row * n_part + p) * 2 + 1] *
+         __expf(ws_ml[(row * n_part + p) * 2] - M);
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  for (int c = threadIdx.x; c < r; c += blockDim.x) {
+    float a = 0.f;
+    for (int p = 0; p < n_part; ++p) {
+      const float w = __expf(ws_ml[(row * n_part + p) * 2] - M);
+      if (w > 0.f) a += ws_acc[(row * n_part + p) * r + c] * w;
+    }
+    out[row * r + c] = a * inv;
+  }
+}
+
+// Which instantiation covers (W, r); 0 = none (caller uses the scalar path).
+int latent_attn_mfma_class(int W, int r) {
+  if (W % 8 != 0) return 0;
+  const int Wp = (W + 31) & ~31, rp = (r + 15) & ~15;
+  if (Wp <= 128 && rp <= 128) return 1;
+  if (Wp <= 320 && rp <= 256) return 2;
+  if (Wp <= 640 && rp <= 512) return 3;
+  return 0;
+}
+
+void launch_latent_attn_mfma(float* out, float* ws_acc, float* ws_ml,
+                             const unsigned short* q,
+                             const unsigned short* cache,
+                             const int* block_tables, const int* cu_q,
+                             const int* seq_lens, int tokens, int n_seqs,
+                             int heads, int r, int rd, int block_size,
+                             int table_width, float scale, int n_part,
+                             hipStream_t st) {
+  if (tokens == 0) return;
+  const int cls = latent_attn_mfma_class(r + rd, r);
+  const int rp = (r + 15) & ~15;
+  int blocks;
+  if (cu_q == nullptr)
+    blocks = n_seqs * ((heads + LM_ROWS - 1) / LM_ROWS);
+  else
+    blocks = (int)(((long)tokens * heads + LM_ROWS - 1) / LM_ROWS) + n_seqs;
+  dim3 grid(blocks, n_part);
+  const size_t lds = (size_t)rp * LM_VS * sizeof(unsigned short);
+#define LM_LAUNCH(KQ, NO)                                                    \
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KQ, NO>), grid, dim3(256), lds, \
+                     st, out, ws_acc, ws_ml, q, cache, block_tables, cu_q,   \
+                     seq_lens, n_seqs, heads, r, rd, block_size, table_width, \
+                     scale, n_part)
+  if (cls == 1) LM_LAUNCH(4, 8);
+  else if (cls == 2) LM_LAUNCH(10, 16);
+  else LM_LAUNCH(20, 32);
+#undef LM_LAUNCH
+  if (n_part > 1)
+    hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens * heads),
+                       dim3(64), 0, st, out, ws_acc, ws_ml, r, n_part);
+}
+
+}  // namespace hyb
+}  // namespace xllm

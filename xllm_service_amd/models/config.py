@@ -199,7 +199,19 @@ def _pugovik_preset(name, width, n_layers, heads, vocab=32000, experts=16,
         norm=dict(eps=1e-6, groups=4), residual_mult=0.5), name=name)
 
 
+def _llama_equal(name, width, n_layers, heads, vocab=32000, ff=None):
+    """Llama stack of the same width, depth and active feed-forward size
+    as the pugovik bench stack of that width (comparison baseline)."""
+    return ModelConfig(name=name, vocab_size=vocab, hidden_size=width,
+                       intermediate_size=ff or width, num_layers=n_layers,
+                       num_heads=heads, num_kv_heads=max(heads // 4, 1),
+                       head_dim=width // heads, rope_theta=10000.0,
+                       max_position=16384)
+
+
 PRESETS.update({
+    "llama-2k": _llama_equal("llama-2k", 2048, 8, 16),
+    "llama-4k": _llama_equal("llama-4k", 4096, 8, 32),
     # CPU-test sized hybrid stack
     "pugovik-tiny": _pugovik_preset("pugovik-tiny", 128, 4, 4, vocab=256,
                                     experts=8, top=2, ff=64, every_attn=2,
