@@ -375,3 +375,81 @@ def test_latent_attn_decode_rows_of_unequal_context(dev, dt, heads, r, rd):
         for h in range(heads):
             _close(out[s, h], _plain_latent_attn(q[s, h], rows, 0.2, r, L),
                    _tol(dt))
+
+
+@pytest.mark.parametrize("dev", DEVS)
+def test_decay_attn_long_portions(dev):
+    """Portions long enough for the chunk-parallel path on the GPU: two
+    sequences in one call, one continuing from a stored state, lengths that
+    end inside a chunk; then a second portion continues both."""
+    heads, d, vd = 2, 16, 24
+    g = torch.Generator().manual_seed(15)
+    lens1, lens2 = [700, 301], [129, 260]
+    T1, T2 = sum(lens1), sum(lens2)
+    wide = torch.randn(T1 + T2, heads * (2 * d + vd), generator=g) * 0.7
+    a = torch.tensor([0.99, 0.8])
+    state = torch.zeros(3, heads, d, vd)
+    state[2] = torch.randn(heads, d, vd, generator=g)
+    init = state.clone()
+    sd, wd, ad = state.to(dev), wide.to(dev), a.to(dev)
+    i32 = dict(dtype=torch.int32, device=dev)
+    o1 = torch.empty(T1, heads, vd, dtype=torch.float32, device=dev)
+    x = wd[:T1]
+    H.decay_attn(x[:, :heads * d], x[:, heads * d:2 * heads * d],
+                 x[:, 2 * heads * d:], ad, sd, torch.tensor([0, 2], **i32),
+                 torch.tensor([0, 700, 1001], **i32),
+                 torch.tensor([0, 5], **i32), o1, max_q_len=700)
+    o2 = torch.empty(T2, heads, vd, dtype=torch.float32, device=dev)
+    x = wd[T1:]
+    H.decay_attn(x[:, :heads * d], x[:, heads * d:2 * heads * d],
+                 x[:, 2 * heads * d:], ad, sd, torch.tensor([0, 2], **i32),
+                 torch.tensor([0, 129, 389], **i32),
+                 torch.tensor([700, 306], **i32), o2, max_q_len=260)
+    seqs = [(torch.cat([wide[:700], wide[T1:T1 + 129]]), 0, False),
+            (torch.cat([wide[700:T1], wide[T1 + 129:]]), 2, True)]
+    got = [torch.cat([o1[:700], o2[:129]]), torch.cat([o1[700:], o2[129:]])]
+    for (x, slot, carried), o in zip(seqs, got):
+        for h in range(heads):
+            S0 = init[slot, h].to(F64) if carried else torch.zeros(d, vd,
+                                                                   dtype=F64)
+            want, S = _plain_decay(
+                x[:, h * d:(h + 1) * d],
+                x[:, heads * d + h * d:heads * d + (h + 1) * d],
+                x[:, 2 * heads * d + h * vd:2 * heads * d + (h + 1) * vd],
+                float(a[h]), S0)
+            _close(o[:, h], want, 5e-5)
+            _close(sd[slot, h], S, 5e-5)
+
+
+@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("skew", [False, True])
+def test_routed_experts_three_execution_shapes_agree(dev, skew):
+    """All-experts batched, padded-by-expert and expert-by-expert execution
+    give the same mixture; `skew` sends most tokens to one expert so the
+    padded shape is refused."""
+    from xllm_service_amd.models.moe import RoutedExperts
+    from hybrid_oracle import o_experts
+    g = torch.Generator().manual_seed(16)
+    W, ff, E, top, T = 24, 10, 8, 2, 150
+    m = RoutedExperts(W, ff, E, top, 4, 2, torch.float32)
+    with torch.no_grad():
+        m.router.copy_(torch.randn(E, W, generator=g) * 0.5)
+        if skew:
+            m.router[0] += 3.0 * torch.ones(W) / math.sqrt(W)
+        m.w_gate_up.copy_(torch.randn(E, 2 * ff, W, generator=g) * 0.3)
+        m.w_down.copy_(torch.randn(E, W, ff, generator=g) * 0.3)
+    h = torch.randn(T, W, generator=g) + (2.0 / math.sqrt(W) if skew else 0.0)
+    wt = {"router": m.router.detach().to(F64)}
+    for e in range(E):
+        wt[f"e{e}.gate"] = m.w_gate_up[e, :ff].detach().to(F64)
+        wt[f"e{e}.up"] = m.w_gate_up[e, ff:].detach().to(F64)
+        wt[f"e{e}.down"] = m.w_down[e].detach().to(F64)
+    fc = dict(router=dict(experts=E, top=top, groups=dict(count=4, keep=2)))
+    want = o_experts(wt, "", fc, h.to(F64))
+    m = m.to(dev)
+    with torch.no_grad():
+        sorted_out = m(h.to(dev))
+        m.dense_max_tokens = 10 ** 6
+        dense_out = m(h.to(dev))
+    _close(sorted_out, want, 2e-5)
+    _close(dense_out, want, 2e-5)

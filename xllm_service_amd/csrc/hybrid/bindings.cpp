@@ -41,7 +41,8 @@ void launch_latent_attn_mfma(float*, float*, float*, const unsigned short*,
 template <typename T>
 void launch_decay_attn(float*, const T*, const T*, const T*, const float*,
                        float*, const int*, const int*, const int*, int, int,
-                       int, int, long, long, long, hipStream_t);
+                       int, int, long, long, long, int, int, float*,
+                       hipStream_t);
 template <typename T>
 void launch_moe_route(int*, float*, const T*, const float*, int, int, int, int,
                       int, int, long, hipStream_t);
@@ -227,8 +228,9 @@ void latent_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables,
       // fill the chip (sizes known on the host only: no sync)
       const int tps = (H + 63) / 64;
       const long max_tiles = ((long)block_tables.size(1) * cache.size(1) + 31) / 32;
-      n_part = (int)std::min<long>(std::min<long>(16, max_tiles),
-                                   std::max<long>(1, 512 / ((long)T * tps)));
+      n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
+                                   std::max<long>(1, 2048 / ((long)T * tps)));
+      n_part = std::max(n_part, 1);
     }
     if (n_part > 1) {
       ws_acc = torch::empty({(long)T * H * n_part, (long)r}, out.options());
@@ -251,9 +253,11 @@ void latent_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables,
 
 // out fp32 [T, H, Dv]; q,k [T, H*D] / v [T, H*Dv] row views (pre-activation)
 // state fp32 [slots, H, D, Dv]; cu_q None => one token per sequence
+// max_q_len: host-side bound on the longest sequence chunk (0 = unknown);
+// long chunks take the chunk-parallel path
 void decay_attn(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
                 Tensor state, Tensor slots, c10::optional<Tensor> cu_q,
-                Tensor ctx_lens) {
+                Tensor ctx_lens, long max_q_len) {
   CHK_F32C(out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_F32C(decay);
   CHK_F32C(state); CHK_I32C(slots); CHK_I32C(ctx_lens);
   TORCH_CHECK(state.dim() == 4 && q.dim() == 2 && k.dim() == 2 &&
@@ -274,10 +278,24 @@ void decay_attn(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
   } else {
     TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
   }
+  int chunk = 128, max_chunks = 1;
+  Tensor ws;
+  if (cu != nullptr) {
+    const long bound = max_q_len > 0 ? std::min<long>(max_q_len, T) : T;
+    const long per_seq = (long)H * D * Dv * 4;
+    while ((bound + chunk - 1) / chunk * n_seqs * per_seq > (1L << 31))
+      chunk *= 2;                             // keep the scratch under 2 GiB
+    if (bound >= 2L * chunk) {
+      max_chunks = (int)((bound + chunk - 1) / chunk);
+      ws = torch::empty({(long)n_seqs * max_chunks, (long)H, (long)D, (long)Dv},
+                        state.options());
+    }
+  }
+  float* wsp = max_chunks > 1 ? ptr<float>(ws) : nullptr;
   if (is_f32(q))
-    hy::launch_decay_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), cur());
+    hy::launch_decay_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), chunk, max_chunks, wsp, cur());
   else
-    hy::launch_decay_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), cur());
+    hy::launch_decay_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), chunk, max_chunks, wsp, cur());
 }
 
 void moe_route(Tensor ids, Tensor wts, Tensor h, Tensor wr, long top,

@@ -11,6 +11,11 @@
 // rows i = r, r+16, ... of column j; a token's output column is the sum over
 // the 16 threads sharing j (a 16-lane shuffle reduction). Tokens are staged
 // through LDS 16 at a time.
+//
+// Long prompt chunks run chunk-parallel: every `chunk` tokens first build
+// their own state from zero (all chunks at once), a scan kernel turns these
+// into the state before each chunk, and a second parallel pass produces the
+// outputs. Same recurrence, re-associated only at chunk edges.
 #include "hybrid_common.h"
 
 namespace xllm {
@@ -27,19 +32,31 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
     const T* __restrict__ v, const float* __restrict__ decay,
     float* __restrict__ state, const int* __restrict__ slots,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int heads,
-    int D, int Dv, long q_stride, long k_stride, long v_stride) {
+    int D, int Dv, long q_stride, long k_stride, long v_stride, int mode,
+    int chunk, int max_chunks, float* __restrict__ ws) {
   extern __shared__ float smem[];
   float* qs = smem;                       // [TC][D]
   float* ks = qs + DA_TC * D;             // [TC][D]
   float* vs = ks + DA_TC * D;             // [TC][VS]
 
-  const int s = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * DA_VS;
+  // mode 0: whole sequence chunk in one workgroup (state slot in and out).
+  // mode 1: tokens [c*chunk, (c+1)*chunk) from a zero state, no outputs;
+  //         the chunk's own state goes to ws[s*max_chunks + c].
+  // mode 2: the same tokens starting from ws[s*max_chunks + c] (filled by
+  //         the scan kernel below), outputs written, no state out.
+  const int s = blockIdx.x / max_chunks, cidx = blockIdx.x % max_chunks;
+  const int h = blockIdx.y, v0 = blockIdx.z * DA_VS;
   const int tid = threadIdx.x;
   const int j = tid / DA_R, r = tid % DA_R;
   const int col = v0 + j;
   const bool col_ok = col < Dv;
-  const int t0 = cu_q ? cu_q[s] : s;
-  const int t1 = cu_q ? cu_q[s + 1] : s + 1;
+  int t0 = cu_q ? cu_q[s] : s;
+  int t1 = cu_q ? cu_q[s + 1] : s + 1;
+  if (mode != 0) {
+    t0 += cidx * chunk;
+    if (t0 >= t1) return;                   // uniform for the workgroup
+    t1 = min(t1, t0 + chunk);
+  }
   const int slot = slots[s];
   const float dec = decay[h];
   const int M = (D + DA_R - 1) / DA_R;
@@ -49,7 +66,12 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
   for (int m = 0; m < DA_MAXM; ++m) S[m] = 0.f;
   float* sp = (slot >= 0)
       ? state + (((long)slot * heads + h) * D) * (long)Dv : nullptr;
-  if (sp && ctx_lens[s] > 0 && col_ok) {
+  bool load = sp && ctx_lens[s] > 0;
+  if (mode != 0) {
+    sp = ws + ((((long)s * max_chunks + cidx) * heads + h) * D) * (long)Dv;
+    load = mode == 2;
+  }
+  if (load && col_ok) {
 #pragma unroll
     for (int m = 0; m < DA_MAXM; ++m) {
       const int i = r + DA_R * m;
@@ -85,12 +107,14 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
           o += S[m] * qs[tt * D + i];
         }
       }
-      o = group_reduce_sum<DA_R>(o);
-      if (r == 0 && col_ok)
-        out[((long)(tb + tt) * heads + h) * Dv + col] = o;
+      if (mode != 1) {
+        o = group_reduce_sum<DA_R>(o);
+        if (r == 0 && col_ok)
+          out[((long)(tb + tt) * heads + h) * Dv + col] = o;
+      }
     }
   }
-  if (sp && col_ok) {
+  if (sp && col_ok && mode != 2) {
 #pragma unroll
     for (int m = 0; m < DA_MAXM; ++m) {
       const int i = r + DA_R * m;
@@ -99,25 +123,75 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
   }
 }
 
+// Sequential pass over a sequence's chunk states (one thread per state
+// element): ws[c] <- state before chunk c; the state after the last chunk
+// goes to the sequence's slot.
+__global__ void decay_scan_kernel(float* __restrict__ ws,
+                                  float* __restrict__ state,
+                                  const float* __restrict__ decay,
+                                  const int* __restrict__ slots,
+                                  const int* __restrict__ cu_q,
+                                  const int* __restrict__ ctx_lens, int heads,
+                                  long per_head, int chunk, int max_chunks) {
+  const int s = blockIdx.y;
+  const long per_seq = per_head * heads;
+  const long e = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (e >= per_seq) return;
+  const int h = (int)(e / per_head);
+  const int qlen = cu_q[s + 1] - cu_q[s];
+  const int n_chunks = (qlen + chunk - 1) / chunk;
+  const int slot = slots[s];
+  const float a = decay[h];
+  float S = (slot >= 0 && ctx_lens[s] > 0) ? state[slot * per_seq + e] : 0.f;
+  const float a_full = powf(a, (float)chunk);
+  for (int c = 0; c < n_chunks; ++c) {
+    float* w = ws + ((long)s * max_chunks + c) * per_seq + e;
+    const float local = *w;
+    *w = S;
+    const int len = min(chunk, qlen - c * chunk);
+    S = (len == chunk ? a_full : powf(a, (float)len)) * S + local;
+  }
+  if (slot >= 0) state[slot * per_seq + e] = S;
+}
+
 template <typename T>
 void launch_decay_attn(float* out, const T* q, const T* k, const T* v,
                        const float* decay, float* state, const int* slots,
                        const int* cu_q, const int* ctx_lens, int n_seqs,
                        int heads, int D, int Dv, long q_stride, long k_stride,
-                       long v_stride, hipStream_t st) {
+                       long v_stride, int chunk, int max_chunks, float* ws,
+                       hipStream_t st) {
   if (n_seqs == 0) return;
-  dim3 grid(n_seqs, heads, (Dv + DA_VS - 1) / DA_VS);
   const size_t lds = (size_t)(2 * DA_TC * D + DA_TC * DA_VS) * sizeof(float);
+  const int vz = (Dv + DA_VS - 1) / DA_VS;
+  if (ws == nullptr || max_chunks <= 1) {
+    hipLaunchKernelGGL((decay_attn_kernel<T>), dim3(n_seqs, heads, vz),
+                       dim3(256), lds, st, out, q, k, v, decay, state, slots,
+                       cu_q, ctx_lens, heads, D, Dv, q_stride, k_stride,
+                       v_stride, 0, 0, 1, nullptr);
+    return;
+  }
+  // chunk-parallel: local chunk states, a short scan, then the outputs
+  dim3 grid(n_seqs * max_chunks, heads, vz);
   hipLaunchKernelGGL((decay_attn_kernel<T>), grid, dim3(256), lds, st, out, q,
                      k, v, decay, state, slots, cu_q, ctx_lens, heads, D, Dv,
-                     q_stride, k_stride, v_stride);
+                     q_stride, k_stride, v_stride, 1, chunk, max_chunks, ws);
+  const long per_head = (long)D * Dv;
+  const long per_seq = per_head * heads;
+  hipLaunchKernelGGL(decay_scan_kernel,
+                     dim3((unsigned)((per_seq + 255) / 256), n_seqs),
+                     dim3(256), 0, st, ws, state, decay, slots, cu_q,
+                     ctx_lens, heads, per_head, chunk, max_chunks);
+  hipLaunchKernelGGL((decay_attn_kernel<T>), grid, dim3(256), lds, st, out, q,
+                     k, v, decay, state, slots, cu_q, ctx_lens, heads, D, Dv,
+                     q_stride, k_stride, v_stride, 2, chunk, max_chunks, ws);
 }
 
 #define INST_DA(T)                                                            \
   template void launch_decay_attn<T>(                                         \
       float*, const T*, const T*, const T*, const float*, float*, const int*, \
-      const int*, const int*, int, int, int, int, long, long, long,           \
-      hipStream_t);
+      const int*, const int*, int, int, int, int, long, long, long, int, int, \
+      float*, hipStream_t);
 INST_DA(float)
 INST_DA(unsigned short)
 

@@ -88,8 +88,12 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   const int* table = block_tables + (long)s * table_width;
 
   // ---- this lane's row -----------------------------------------------------
-  const int rho = row0 + wv * 16 + n;
-  const bool wave_on = row0 + wv * 16 < rows_in_seq;
+  // col_split: a token with at most 16 heads has one 16-row tile; instead of
+  // idling three waves, all four score it and each owns every fourth
+  // 16-column tile of the output
+  const bool col_split = rows_in_seq <= 16;
+  const int rho = row0 + (col_split ? 0 : wv * 16) + n;
+  const bool wave_on = col_split || row0 + wv * 16 < rows_in_seq;
   const bool row_ok = rho < rows_in_seq;
   const int limit = row_ok ? ctx + rho / heads + 1 : 0;
   const long grow = (long)q0 * heads + rho;          // row in [T*H]
@@ -183,7 +187,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     }
 #pragma unroll
     for (int no = 0; no < NO; ++no) {
-      if (no * 16 < rp) {
+      if (no * 16 < rp && (!col_split || (no & 3) == wv)) {
         acc[no] *= alpha;
         const bf16x8 a = ld8(vt + (no * 16 + n) * LM_VS + g * 8);
         acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, acc[no], 0, 0, 0);
@@ -202,7 +206,8 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r) orow[col] = acc[no][rr] * inv;
+        if (no * 16 < rp && col < r && (!col_split || (no & 3) == wv))
+          orow[col] = acc[no][rr] * inv;
       }
   } else {
     // partials are indexed by the OUTPUT row: [row][part]
@@ -213,9 +218,12 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r) arow[col] = acc[no][rr];
+        if (no * 16 < rp && col < r && (!col_split || (no & 3) == wv))
+          arow[col] = acc[no][rr];
       }
-    if (g == 0) { ws_ml[base * 2] = m; ws_ml[base * 2 + 1] = l; }
+    if (g == 0 && (!col_split || wv == 0)) {
+      ws_ml[base * 2] = m; ws_ml[base * 2 + 1] = l;
+    }
   }
 }
 

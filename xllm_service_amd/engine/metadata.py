@@ -39,6 +39,7 @@ class AttnMetadata:
     prefill_ctx_lens: Optional[torch.Tensor] = None      # [n_prefill] int32
     prefill_state_slots: Optional[torch.Tensor] = None   # [n_prefill] int32
     decode_state_slots: Optional[torch.Tensor] = None    # [n_decode] int32
+    max_prefill_len: int = 0      # longest prefill chunk (host int, 0 = n/a)
 
     @property
     def num_tokens(self) -> int:

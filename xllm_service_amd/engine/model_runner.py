@@ -253,6 +253,8 @@ class ModelRunner:
         if self.uses_state_slots:
             i32 = dict(dtype=torch.int32, device=dev)
             if plan.prefills:
+                meta.max_prefill_len = max(sp.chunk_len
+                                           for sp in plan.prefills)
                 meta.prefill_ctx_lens = torch.tensor(p_ctx, **i32)
                 meta.prefill_state_slots = torch.tensor(p_state, **i32)
             if plan.decodes:

@@ -153,7 +153,8 @@ class DecayLinearAttention(nn.Module):
         if np_:
             hops.decay_attn(q[:np_], k[:np_], v[:np_], self.decay, state,
                             meta.prefill_state_slots, meta.cu_q,
-                            meta.prefill_ctx_lens, o[:np_])
+                            meta.prefill_ctx_lens, o[:np_],
+                            max_q_len=meta.max_prefill_len)
         if nd:
             hops.decay_attn(q[np_:], k[np_:], v[np_:], self.decay, state,
                             meta.decode_state_slots, None,

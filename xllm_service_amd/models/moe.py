@@ -11,7 +11,8 @@ kernel: few tokens (decode batches, graph capture) run every expert as one
 batched GEMM over all tokens — at those sizes the step is bound by reading
 the expert weights, which a token-sorted pass would read as well, and it
 needs no host round trip; many tokens are sorted by expert and each expert
-multiplies only its own rows.
+multiplies only its own rows (as one padded batched GEMM when the load is
+near-even, expert by expert otherwise).
 """
 from __future__ import annotations
 
@@ -54,7 +55,26 @@ class RoutedExperts(nn.Module):
             return hops.moe_combine(y, rows, wts, T)
         flat = ids.reshape(-1).long()
         order = torch.argsort(flat, stable=True)
-        counts = torch.bincount(flat, minlength=self.experts).tolist()
+        counts_t = torch.bincount(flat, minlength=self.experts)
+        counts = counts_t.tolist()                 # the one host round trip
+        cap, total = max(counts), T * self.top
+        if cap * self.experts <= 1.5 * total + 16 * self.experts:
+            # near-even load: pad every expert to `cap` rows and run all of
+            # them as two batched GEMMs
+            e_sorted = flat[order]
+            starts = torch.cumsum(counts_t, 0) - counts_t
+            dest = e_sorted * cap + (torch.arange(total, device=h.device)
+                                     - starts[e_sorted])
+            xs = h.new_zeros(self.experts * cap, self.width)
+            xs[dest] = h[order // self.top]
+            gu = torch.bmm(xs.view(self.experts, cap, self.width),
+                           self.w_gate_up.transpose(1, 2))
+            y = torch.bmm(hops.silu_mul(gu), self.w_down.transpose(1, 2))
+            rows = torch.empty_like(dest)
+            rows[order] = dest
+            return hops.moe_combine(y.view(-1, self.width),
+                                    rows.view(T, self.top).to(torch.int32),
+                                    wts, T)
         xs = h[order // self.top]
         ys = torch.empty(T * self.top, self.width, dtype=h.dtype,
                          device=h.device)

@@ -106,11 +106,14 @@ def latent_attn(q, cache, block_tables, cu_q, seq_lens, scale, kv_rank, out):
     return out
 
 
-def decay_attn(q, k, v, decay, state, slots, cu_q, ctx_lens, out):
+def decay_attn(q, k, v, decay, state, slots, cu_q, ctx_lens, out,
+               max_q_len: int = 0):
     """out fp32 [T, H, Dv] (written); q/k/v are pre-activation row views
-    [T, H*D] / [T, H*Dv]; state fp32 [slots, H, D, Dv] updated in place."""
+    [T, H*D] / [T, H*Dv]; state fp32 [slots, H, D, Dv] updated in place.
+    max_q_len: host-known bound on the longest sequence chunk (0: unknown)."""
     if q.is_cuda:
-        _hyb().decay_attn(out, q, k, v, decay, state, slots, cu_q, ctx_lens)
+        _hyb().decay_attn(out, q, k, v, decay, state, slots, cu_q, ctx_lens,
+                          max_q_len)
         return out
     H, D, Dv = state.shape[1:]
     T = q.shape[0]
