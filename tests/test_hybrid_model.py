@@ -138,7 +138,7 @@ def test_layers_residual_stream(root, target, name):
         if target[1] == torch.float32:
             assert float(err.max()) < 2e-4, (name, i, float(err.max()))
         else:
-            assert float(err.median()) < 0.05, (name, i, err)
+            assert float(err.median()) < 0.1, (name, i, err)
 
 
 @pytest.mark.parametrize("target", TARGETS)

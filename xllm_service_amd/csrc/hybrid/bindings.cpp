@@ -43,9 +43,8 @@ void launch_decay_attn(float*, const T*, const T*, const T*, const float*,
                        float*, const int*, const int*, const int*, int, int,
                        int, int, long, long, long, int, int, float*,
                        hipStream_t);
-template <typename T>
-void launch_moe_route(int*, float*, const T*, const float*, int, int, int, int,
-                      int, int, long, hipStream_t);
+void launch_moe_route(int*, float*, const float*, int, int, int, int, int,
+                      hipStream_t);
 template <typename T>
 void launch_moe_combine(float*, const T*, const int*, const float*, long, int,
                         int, hipStream_t);
@@ -298,21 +297,19 @@ void decay_attn(Tensor out, Tensor q, Tensor k, Tensor v, Tensor decay,
     hy::launch_decay_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<float>(decay), ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, D, Dv, q.stride(0), k.stride(0), v.stride(0), chunk, max_chunks, wsp, cur());
 }
 
-void moe_route(Tensor ids, Tensor wts, Tensor h, Tensor wr, long top,
-               long n_groups, long keep) {
-  CHK_I32C(ids); CHK_F32C(wts); CHK_ACT(h); CHK_F32C(wr);
-  TORCH_CHECK(h.dim() == 2 && wr.dim() == 2);
-  const int T = h.size(0), width = h.size(1), E = wr.size(0);
-  TORCH_CHECK(wr.size(1) == width && ids.numel() == (long)T * top &&
-              wts.numel() == (long)T * top);
+// z fp32 [T, E] router logits -> ids int32 [T, top], wts fp32 [T, top]
+void moe_route(Tensor ids, Tensor wts, Tensor z, long top, long n_groups,
+               long keep) {
+  CHK_I32C(ids); CHK_F32C(wts); CHK_F32C(z);
+  TORCH_CHECK(z.dim() == 2);
+  const int T = z.size(0), E = z.size(1);
+  TORCH_CHECK(ids.numel() == (long)T * top && wts.numel() == (long)T * top);
   TORCH_CHECK(top >= 1 && top <= E && n_groups >= 1 && E % n_groups == 0 &&
               keep >= 1 && keep <= n_groups &&
               keep * (E / n_groups) >= top, "bad routing constants");
   TORCH_CHECK((2 * E + n_groups) * 4 <= 64 * 1024, "too many experts");
-  if (is_f32(h))
-    hy::launch_moe_route<float>(ptr<int>(ids), ptr<float>(wts), ptr<float>(h), ptr<float>(wr), T, width, E, top, n_groups, keep, h.stride(0), cur());
-  else
-    hy::launch_moe_route<bf>(ptr<int>(ids), ptr<float>(wts), ptr<bf>(h), ptr<float>(wr), T, width, E, top, n_groups, keep, h.stride(0), cur());
+  hy::launch_moe_route(ptr<int>(ids), ptr<float>(wts), ptr<float>(z), T, E,
+                       top, n_groups, keep, cur());
 }
 
 // out fp32 [T, width]; y [R, width] contiguous; rows int32 [T, top] < R

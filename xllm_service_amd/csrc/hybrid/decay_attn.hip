@@ -71,11 +71,32 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
     sp = ws + ((((long)s * max_chunks + cidx) * heads + h) * D) * (long)Dv;
     load = mode == 2;
   }
-  if (load && col_ok) {
+  // The 16-column slice of the state is 64 B per row: move it with float4
+  // accesses (a wave covers 16 whole rows) through an LDS tile instead of
+  // one 4 B element per lane and row.
+  float* tile = smem;                     // [D][DA_VS + 1], reused by staging
+  const bool vec_ok = (Dv % 4 == 0) && (v0 + DA_VS <= Dv);
+  if (load) {
+    if (vec_ok) {
+      for (int idx = tid; idx < D * 4; idx += 256) {
+        const int i = idx >> 2, c4 = (idx & 3) * 4;
+        const float4 x = *reinterpret_cast<const float4*>(
+            sp + (long)i * Dv + v0 + c4);
+        float* d = tile + i * (DA_VS + 1) + c4;
+        d[0] = x.x; d[1] = x.y; d[2] = x.z; d[3] = x.w;
+      }
+      __syncthreads();
 #pragma unroll
-    for (int m = 0; m < DA_MAXM; ++m) {
-      const int i = r + DA_R * m;
-      if (m < M && i < D) S[m] = sp[(long)i * Dv + col];
+      for (int m = 0; m < DA_MAXM; ++m) {
+        const int i = r + DA_R * m;
+        if (m < M && i < D) S[m] = tile[i * (DA_VS + 1) + j];
+      }
+    } else if (col_ok) {
+#pragma unroll
+      for (int m = 0; m < DA_MAXM; ++m) {
+        const int i = r + DA_R * m;
+        if (m < M && i < D) S[m] = sp[(long)i * Dv + col];
+      }
     }
   }
 
@@ -114,11 +135,27 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
       }
     }
   }
-  if (sp && col_ok && mode != 2) {
+  if (sp && mode != 2) {
+    if (vec_ok) {
+      __syncthreads();                    // staging buffers are done with
 #pragma unroll
-    for (int m = 0; m < DA_MAXM; ++m) {
-      const int i = r + DA_R * m;
-      if (m < M && i < D) sp[(long)i * Dv + col] = S[m];
+      for (int m = 0; m < DA_MAXM; ++m) {
+        const int i = r + DA_R * m;
+        if (m < M && i < D) tile[i * (DA_VS + 1) + j] = S[m];
+      }
+      __syncthreads();
+      for (int idx = tid; idx < D * 4; idx += 256) {
+        const int i = idx >> 2, c4 = (idx & 3) * 4;
+        const float* d = tile + i * (DA_VS + 1) + c4;
+        *reinterpret_cast<float4*>(sp + (long)i * Dv + v0 + c4) =
+            make_float4(d[0], d[1], d[2], d[3]);
+      }
+    } else if (col_ok) {
+#pragma unroll
+      for (int m = 0; m < DA_MAXM; ++m) {
+        const int i = r + DA_R * m;
+        if (m < M && i < D) sp[(long)i * Dv + col] = S[m];
+      }
     }
   }
 }

@@ -11,15 +11,21 @@
 //                                              in registers for the whole kernel
 //   online softmax per row in fp32 (a lane holds 8 keys of ONE row)
 //   O^T[col][row] += V^T[col][key] P^T[key][row]
-//                                              A = V^T from LDS (the tile is
-//                                              staged transposed once per
-//                                              workgroup), B = the lane's own 8
+//                                              A = V^T by hardware transpose
+//                                              reads (ds_read_b64_tr_b16) of the
+//                                              tile staged in LDS with plain
+//                                              16 B writes; B = the lane's own 8
 //                                              weights: no exchange needed
-// The C layout of S^T hands each lane keys g*4+r of both 16-key halves; the
-// staged V^T stores key columns in exactly that order, so P never moves.
-// Softmax weights stay 32-bit: p is split exactly into three bf16 terms
-// (8+8+8 mantissa bits) and each term gets its own MFMA into the fp32
+// The C layout of S^T hands a lane rows g*4+r of both 16-row halves; feeding
+// key k0 + (m>>2)*8 + half*4 + (m&3) as A row m makes those the keys
+// g*8 .. g*8+7 in natural order, which is what the transposed V fragment
+// holds. Softmax weights stay 32-bit: p is split exactly into three bf16
+// terms (8+8+8 mantissa bits) and each term gets its own MFMA into the fp32
 // accumulator.
+//
+// LDS image of a 32-key tile, per 16-column tile `nt` (512 bf16): element
+// (k, d) at nt*512 + ((k>>2)&1)*256 + (k>>3)*64 + (k&3)*16 + (d&15); a lane
+// reads 8 B at g*128 + n*8 (bytes) of each 512-byte half.
 //
 // Decode splits the context over `n_part` workgroups per token; partial
 // (acc, max, sum) triples are merged by a second small kernel.
@@ -36,7 +42,6 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 constexpr int LM_ROWS = 64;     // rows per workgroup
 constexpr int LM_KT = 32;       // keys per tile
-constexpr int LM_VS = 40;       // V^T row stride in LDS (32 keys + pad)
 
 struct alignas(16) u16x8 { unsigned short x[8]; };
 
@@ -52,7 +57,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_seqs, int heads, int r, int rd,
     int block_size, int table_width, float scale, int n_part) {
-  extern __shared__ unsigned short vt[];          // [rp][LM_VS]
+  extern __shared__ unsigned short vt[];          // tr16 image, see above
   const int W = r + rd;
   const int Wp = (W + 31) & ~31;
   const int rp = (r + 15) & ~15;
@@ -90,7 +95,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   // ---- this lane's row -----------------------------------------------------
   // col_split: a token with at most 16 heads has one 16-row tile; instead of
   // idling three waves, all four score it and each owns every fourth
-  // 16-column tile of the output
+  // 64-column batch of the output
   const bool col_split = rows_in_seq <= 16;
   const int rho = row0 + (col_split ? 0 : wv * 16) + n;
   const bool wave_on = col_split || row0 + wv * 16 < rows_in_seq;
@@ -114,8 +119,8 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   for (int t = t_begin; t < t_end; ++t) {
     const int k0 = t * LM_KT;
     __syncthreads();
-    // stage V^T (first rp columns of each cached row), keys permuted so
-    // that position g*8 + j holds key g*4 + j (j<4) / 16 + g*4 + j-4
+    // stage the first rp columns of each cached row into the tr16 image:
+    // a 16 B chunk (8 columns of one key) stays contiguous
     for (int c = tid; c < LM_KT * CH; c += 256) {
       const int kl = c / CH, part = c - kl * CH;
       const int key = k0 + kl, col = part * 8;
@@ -125,10 +130,9 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
         v8 = *reinterpret_cast<const u16x8*>(
             cache + (blk * block_size + key % block_size) * (long)W + col);
       }
-      const int half = kl >> 4, k16 = kl & 15;
-      const int pos = (k16 >> 2) * 8 + half * 4 + (k16 & 3);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(col + e) * LM_VS + pos] = v8.x[e];
+      *reinterpret_cast<u16x8*>(
+          vt + (col >> 4) * 512 + ((kl >> 2) & 1) * 256 + (kl >> 3) * 64 +
+          (kl & 3) * 16 + (col & 15)) = v8;
     }
     __syncthreads();
     if (!wave_on) continue;
@@ -136,7 +140,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     float sc[8];
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
-      const int key = k0 + h2 * 16 + n;              // A row of this lane
+      const int key = k0 + (n >> 2) * 8 + h2 * 4 + (n & 3);   // A row n
       const bool kok = key < kmax;
       const unsigned short* krow = cache;
       if (kok) {
@@ -156,7 +160,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
       }
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int kk = k0 + h2 * 16 + g * 4 + rr;    // C row = key
+        const int kk = k0 + g * 8 + h2 * 4 + rr;     // key of C row g*4+rr
         sc[h2 * 4 + rr] = (kk < limit) ? sacc[rr] * scale : -INFINITY;
       }
     }
@@ -185,14 +189,44 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
       const float r2 = r1 - bf16_to_f32(h2);
       b1[i] = (short)h1; b2[i] = (short)h2; b3[i] = (short)f32_to_bf16(r2);
     }
+    // four 16-column tiles per batch: 8 transpose reads, then 12 MFMAs
+    const unsigned vbase = (unsigned)(unsigned long long)(vt) +
+                           (unsigned)(g * 128 + n * 8);
 #pragma unroll
-    for (int no = 0; no < NO; ++no) {
-      if (no * 16 < rp && (!col_split || (no & 3) == wv)) {
-        acc[no] *= alpha;
-        const bf16x8 a = ld8(vt + (no * 16 + n) * LM_VS + g * 8);
-        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, acc[no], 0, 0, 0);
-        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, acc[no], 0, 0, 0);
-        acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b3, acc[no], 0, 0, 0);
+    for (int nb = 0; nb < NO / 4; ++nb) {
+      if (nb * 64 < rp && (!col_split || (nb & 3) == wv)) {
+        typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
+        u32x2 tr[8];
+        const unsigned va = vbase + (unsigned)(nb * 4096);
+        asm volatile(
+            "ds_read_b64_tr_b16 %[t0], %[a] offset:0\n\t"
+            "ds_read_b64_tr_b16 %[t1], %[a] offset:512\n\t"
+            "ds_read_b64_tr_b16 %[t2], %[a] offset:1024\n\t"
+            "ds_read_b64_tr_b16 %[t3], %[a] offset:1536\n\t"
+            "ds_read_b64_tr_b16 %[t4], %[a] offset:2048\n\t"
+            "ds_read_b64_tr_b16 %[t5], %[a] offset:2560\n\t"
+            "ds_read_b64_tr_b16 %[t6], %[a] offset:3072\n\t"
+            "ds_read_b64_tr_b16 %[t7], %[a] offset:3584\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : [t0] "=&v"(tr[0]), [t1] "=&v"(tr[1]), [t2] "=&v"(tr[2]),
+              [t3] "=&v"(tr[3]), [t4] "=&v"(tr[4]), [t5] "=&v"(tr[5]),
+              [t6] "=&v"(tr[6]), [t7] "=&v"(tr[7])
+            : [a] "v"(va)
+            : "memory");
+#pragma unroll
+        for (int nn = 0; nn < 4; ++nn) {
+          const int no = nb * 4 + nn;
+          bf16x8 a;
+          unsigned* aw = reinterpret_cast<unsigned*>(&a);
+          aw[0] = tr[2 * nn][0];
+          aw[1] = tr[2 * nn][1];
+          aw[2] = tr[2 * nn + 1][0];
+          aw[3] = tr[2 * nn + 1][1];
+          acc[no] *= alpha;
+          acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b1, acc[no], 0, 0, 0);
+          acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b2, acc[no], 0, 0, 0);
+          acc[no] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b3, acc[no], 0, 0, 0);
+        }
       }
     }
   }
@@ -206,7 +240,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r && (!col_split || (no & 3) == wv))
+        if (no * 16 < rp && col < r && (!col_split || ((no >> 2) & 3) == wv))
           orow[col] = acc[no][rr] * inv;
       }
   } else {
@@ -218,7 +252,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r && (!col_split || (no & 3) == wv))
+        if (no * 16 < rp && col < r && (!col_split || ((no >> 2) & 3) == wv))
           arow[col] = acc[no][rr];
       }
     if (g == 0 && (!col_split || wv == 0)) {
@@ -228,27 +262,32 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
 }
 
 // out[row] = sum_p acc[row][p] e^(m_p - M) / sum_p l_p e^(m_p - M)
-__global__ void latent_attn_merge_kernel(float* __restrict__ out,
-                                         const float* __restrict__ ws_acc,
-                                         const float* __restrict__ ws_ml,
-                                         int r, int n_part) {
+// One workgroup per row; the n_part (<= 64) weights are computed once by the
+// first wave and shared through LDS, the column sums then run over
+// independent loads.
+__global__ void __launch_bounds__(256) latent_attn_merge_kernel(
+    float* __restrict__ out, const float* __restrict__ ws_acc,
+    const float* __restrict__ ws_ml, int r, int n_part) {
+  __shared__ float wgt[64];
   const long row = blockIdx.x;
-  float M = -INFINITY;
-  for (int p = 0; p < n_part; ++p)
-    M = fmaxf(M, ws_ml[(row * n_part + p) * 2]);
-  if (M == -INFINITY) M = 0.f;
-  float L = 0.f;
-  for (int p = 0; p < n_part; ++p)
-    L += ws_ml[(row * n_part + p) * 2 + 1] *
-         __expf(ws_ml[(row * n_part + p) * 2] - M);
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
-  for (int c = threadIdx.x; c < r; c += blockDim.x) {
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    const bool on = tid < n_part;
+    const float mp = on ? ws_ml[(row * n_part + tid) * 2] : -INFINITY;
+    const float lp = on ? ws_ml[(row * n_part + tid) * 2 + 1] : 0.f;
+    float M = wave_reduce_max(mp);
+    if (M == -INFINITY) M = 0.f;
+    const float e = on ? __expf(mp - M) : 0.f;
+    const float L = wave_reduce_sum(lp * e);
+    wgt[tid] = (L > 0.f) ? e / L : 0.f;
+  }
+  __syncthreads();
+  const float* base = ws_acc + row * n_part * (long)r;
+  for (int c = tid; c < r; c += 256) {
     float a = 0.f;
-    for (int p = 0; p < n_part; ++p) {
-      const float w = __expf(ws_ml[(row * n_part + p) * 2] - M);
-      if (w > 0.f) a += ws_acc[(row * n_part + p) * r + c] * w;
-    }
-    out[row * r + c] = a * inv;
+#pragma unroll 8
+    for (int p = 0; p < n_part; ++p) a += base[(long)p * r + c] * wgt[p];
+    out[row * r + c] = a;
   }
 }
 
@@ -279,7 +318,8 @@ void launch_latent_attn_mfma(float* out, float* ws_acc, float* ws_ml,
   else
     blocks = (int)(((long)tokens * heads + LM_ROWS - 1) / LM_ROWS) + n_seqs;
   dim3 grid(blocks, n_part);
-  const size_t lds = (size_t)rp * LM_VS * sizeof(unsigned short);
+  // whole batches of four 16-column tiles (4096 B each)
+  const size_t lds = (size_t)((rp + 63) / 64) * 4096;
 #define LM_LAUNCH(KQ, NO)                                                    \
   hipLaunchKernelGGL((latent_attn_mfma_kernel<KQ, NO>), grid, dim3(256), lds, \
                      st, out, ws_acc, ws_ml, q, cache, block_tables, cu_q,   \
@@ -291,7 +331,7 @@ void launch_latent_attn_mfma(float* out, float* ws_acc, float* ws_ml,
 #undef LM_LAUNCH
   if (n_part > 1)
     hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens * heads),
-                       dim3(64), 0, st, out, ws_acc, ws_ml, r, n_part);
+                       dim3(256), 0, st, out, ws_acc, ws_ml, r, n_part);
 }
 
 }  // namespace hyb

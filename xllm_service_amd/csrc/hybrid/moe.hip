@@ -1,37 +1,28 @@
-// Routed-expert support kernels: the router (fp32 logits, sigmoid scores,
-// group-limited top-k) and the weighted combine of expert outputs. The
+// Routed-expert support kernels: the router's selection (sigmoid scores,
+// group-limited top-k over fp32 logits) and the weighted combine of expert outputs. The
 // expert matrix products themselves are library GEMMs.
 #include "hybrid_common.h"
 
 namespace xllm {
 namespace hyb {
 
-// One wavefront per token. scores[e] = sigmoid(h . Wr[e]) in fp32.
+// One wavefront per token; z [T, E] are the fp32 router logits (an fp32 GEMM
+// upstream), scores = sigmoid(z).
 // Experts form n_groups equal neighbouring groups; a group's score is the
 // sum of its two largest scores; only the `keep` best groups are eligible.
 // ids/weights [T, top]: the eligible experts with the largest scores, weights
 // are the raw scores. Ties go to the lower index.
-template <typename T>
 __global__ void moe_route_kernel(int* __restrict__ ids,
                                  float* __restrict__ wts,
-                                 const T* __restrict__ h,
-                                 const float* __restrict__ wr, int width,
-                                 int E, int top, int n_groups, int keep,
-                                 long h_stride) {
+                                 const float* __restrict__ z, int E, int top,
+                                 int n_groups, int keep) {
   extern __shared__ float smem[];
   float* sc = smem;                 // [E] scores
   float* el = sc + E;               // [E] eligible score or -1 (taken/masked)
   float* gsc = el + E;              // [n_groups]
   const int t = blockIdx.x;
   const int lane = threadIdx.x;
-  const T* hr = h + (long)t * h_stride;
-  for (int e = 0; e < E; ++e) {
-    float d = 0.f;
-    const float* w = wr + (long)e * width;
-    for (int i = lane; i < width; i += 64) d += IO<T>::ld(hr + i) * w[i];
-    d = wave_reduce_sum(d);
-    if (lane == 0) sc[e] = sigmoidf_(d);
-  }
+  for (int e = lane; e < E; e += 64) sc[e] = sigmoidf_(z[(long)t * E + e]);
   __syncthreads();
   const int gsz = E / n_groups;
   if (n_groups > 1) {
@@ -101,14 +92,12 @@ __global__ void moe_combine_kernel(float* __restrict__ out,
   }
 }
 
-template <typename T>
-void launch_moe_route(int* ids, float* wts, const T* h, const float* wr,
-                      int tokens, int width, int E, int top, int n_groups,
-                      int keep, long h_stride, hipStream_t st) {
+void launch_moe_route(int* ids, float* wts, const float* z, int tokens, int E,
+                      int top, int n_groups, int keep, hipStream_t st) {
   if (tokens == 0) return;
   const size_t lds = (size_t)(2 * E + n_groups) * sizeof(float);
-  hipLaunchKernelGGL((moe_route_kernel<T>), dim3(tokens), dim3(64), lds, st,
-                     ids, wts, h, wr, width, E, top, n_groups, keep, h_stride);
+  hipLaunchKernelGGL(moe_route_kernel, dim3(tokens), dim3(64), lds, st, ids,
+                     wts, z, E, top, n_groups, keep);
 }
 
 template <typename T>
@@ -123,9 +112,6 @@ void launch_moe_combine(float* out, const T* y, const int* rows,
 }
 
 #define INST_MOE(T)                                                          \
-  template void launch_moe_route<T>(int*, float*, const T*, const float*,    \
-                                    int, int, int, int, int, int, long,      \
-                                    hipStream_t);                            \
   template void launch_moe_combine<T>(float*, const T*, const int*,          \
                                       const float*, long, int, int,          \
                                       hipStream_t);

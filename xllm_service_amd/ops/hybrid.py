@@ -126,11 +126,15 @@ def decay_attn(q, k, v, decay, state, slots, cu_q, ctx_lens, out,
 
 
 def moe_route(h, w_router, top: int, n_groups: int, keep: int):
+    """Router: fp32 logits h @ w_router^T (a true-fp32 library GEMM on the
+    GPU; h enters as stored, i.e. possibly bf16-rounded), then sigmoid
+    scores and the group-limited top-k selection kernel."""
     if h.is_cuda:
         T = h.shape[0]
+        z = torch.matmul(h.float(), w_router.t())
         ids = torch.empty(T, top, dtype=torch.int32, device=h.device)
         wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
-        _hyb().moe_route(ids, wts, h, w_router, top, n_groups, keep)
+        _hyb().moe_route(ids, wts, z, top, n_groups, keep)
         return ids, wts
     return ref.moe_route(h, w_router, top, n_groups, keep)
 
