@@ -7,6 +7,7 @@
 #include <ATen/hip/HIPContext.h>
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace xllm {
 namespace hyb {
@@ -225,11 +226,16 @@ void latent_attn(Tensor out, Tensor q, Tensor cache, Tensor block_tables,
     if (cu == nullptr) {
       // decode: split the context over workgroups when tokens alone do not
       // fill the chip (sizes known on the host only: no sync)
+      // about one workgroup per CU measured best (batch 8/32/128 at 1k-4k
+      // context): more parts only add fp32 partials to write and merge
       const int tps = (H + 63) / 64;
       const long max_tiles = ((long)block_tables.size(1) * cache.size(1) + 31) / 32;
       n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
-                                   std::max<long>(1, 2048 / ((long)T * tps)));
+                                   std::max<long>(1, 256 / ((long)T * tps)));
       n_part = std::max(n_part, 1);
+      // tuning knob: fixed partition count (1..32)
+      if (const char* e = std::getenv("XLLM_LATENT_PARTS"))
+        n_part = std::min(32, std::max(1, std::atoi(e)));
     }
     if (n_part > 1) {
       ws_acc = torch::empty({(long)T * H * n_part, (long)r}, out.options());

@@ -6,8 +6,8 @@
 // query tensor. A workgroup (4 waves) owns 64 such rows, a wave 16.
 //
 // Per 32-key tile:
-//   S^T[key][row] = K[key][:] . Q[row][:]      A = K rows, 16 B per lane straight
-//                                              from the paged cache; B = Q, held
+//   S^T[key][row] = K[key][:] . Q[row][:]      A = K rows, 16 B per lane from the
+//                                              tile staged in LDS; B = Q, held
 //                                              in registers for the whole kernel
 //   online softmax per row in fp32 (a lane holds 8 keys of ONE row)
 //   O^T[col][row] += V^T[col][key] P^T[key][row]
@@ -40,7 +40,6 @@ namespace hyb {
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
-constexpr int LM_ROWS = 64;     // rows per workgroup
 constexpr int LM_KT = 32;       // keys per tile
 
 struct alignas(16) u16x8 { unsigned short x[8]; };
@@ -49,7 +48,12 @@ XLLM_DEV bf16x8 ld8(const unsigned short* p) {
   return *reinterpret_cast<const bf16x8*>(p);
 }
 
-template <int KQ, int NO>
+// CS = column split: the 4 waves of a workgroup form 4/CS row tiles, and CS
+// waves share one row tile, each owning every CS-th 64-column batch of the
+// output. CS > 1 is for decode (few rows per token): accumulators shrink by
+// CS, which makes room to prefetch the next key tile into registers while
+// the current one is computed.
+template <int KQ, int NO, int CS>
 __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     float* __restrict__ out, float* __restrict__ ws_acc,
     float* __restrict__ ws_ml, const unsigned short* __restrict__ q,
@@ -58,6 +62,13 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     const int* __restrict__ seq_lens, int n_seqs, int heads, int r, int rd,
     int block_size, int table_width, float scale, int n_part) {
   extern __shared__ unsigned short vt[];          // tr16 image, see above
+  __shared__ int tbl[512];                        // block ids of this key range
+  constexpr int RT = 4 / CS;                      // row tiles per workgroup
+  constexpr int ROWS_WG = 16 * RT;
+  constexpr int NB = NO / 4;                      // 64-column batches
+  constexpr int NBL = (NB + CS - 1) / CS;         // ... owned by one wave
+  constexpr int NPF = (KQ + 1) / 2;               // 16 B chunks per thread/tile
+  constexpr bool PF = CS > 1;
   const int W = r + rd;
   const int Wp = (W + 31) & ~31;
   const int rp = (r + 15) & ~15;
@@ -68,13 +79,13 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   int s, lt, qlen, q0;
   const int bid = blockIdx.x;
   if (cu_q == nullptr) {
-    const int tps = (heads + LM_ROWS - 1) / LM_ROWS;
+    const int tps = (heads + ROWS_WG - 1) / ROWS_WG;
     s = bid / tps; lt = bid - s * tps; qlen = 1; q0 = s;
     if (s >= n_seqs) return;
   } else {
     int acc = 0; s = -1; lt = 0;
     for (int i = 0; i < n_seqs; ++i) {
-      const int nt = ((cu_q[i + 1] - cu_q[i]) * heads + LM_ROWS - 1) / LM_ROWS;
+      const int nt = ((cu_q[i + 1] - cu_q[i]) * heads + ROWS_WG - 1) / ROWS_WG;
       if (bid < acc + nt) { s = i; lt = bid - acc; break; }
       acc += nt;
     }
@@ -83,8 +94,8 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   }
   const int rows_in_seq = qlen * heads;
   const int ctx = seq_lens[s] - qlen;
-  const int row0 = lt * LM_ROWS;
-  const int last_row = min(row0 + LM_ROWS, rows_in_seq) - 1;
+  const int row0 = lt * ROWS_WG;
+  const int last_row = min(row0 + ROWS_WG, rows_in_seq) - 1;
   const int kmax = ctx + last_row / heads + 1;       // keys any row here sees
   const int n_tiles = (kmax + LM_KT - 1) / LM_KT;
   const int tpp = (n_tiles + n_part - 1) / n_part;
@@ -93,12 +104,9 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
   const int* table = block_tables + (long)s * table_width;
 
   // ---- this lane's row -----------------------------------------------------
-  // col_split: a token with at most 16 heads has one 16-row tile; instead of
-  // idling three waves, all four score it and each owns every fourth
-  // 64-column batch of the output
-  const bool col_split = rows_in_seq <= 16;
-  const int rho = row0 + (col_split ? 0 : wv * 16) + n;
-  const bool wave_on = col_split || row0 + wv * 16 < rows_in_seq;
+  const int rt = wv % RT, cpart = wv / RT;
+  const int rho = row0 + rt * 16 + n;
+  const bool wave_on = row0 + rt * 16 < rows_in_seq;
   const bool row_ok = rho < rows_in_seq;
   const int limit = row_ok ? ctx + rho / heads + 1 : 0;
   const long grow = (long)q0 * heads + rho;          // row in [T*H]
@@ -110,50 +118,82 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
     qf[kc] = (row_ok && col < W) ? ld8(q + grow * W + col) : z;
   }
-  f32x4 acc[NO];
+  f32x4 acc[NBL * 4];
 #pragma unroll
-  for (int i = 0; i < NO; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < NBL * 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  const int CH = rp >> 3;                            // 16 B chunks per row
-  for (int t = t_begin; t < t_end; ++t) {
-    const int k0 = t * LM_KT;
-    __syncthreads();
-    // stage the first rp columns of each cached row into the tr16 image:
-    // a 16 B chunk (8 columns of one key) stays contiguous
-    for (int c = tid; c < LM_KT * CH; c += 256) {
-      const int kl = c / CH, part = c - kl * CH;
-      const int key = k0 + kl, col = part * 8;
-      u16x8 v8 = {{0, 0, 0, 0, 0, 0, 0, 0}};
+  const int CH = Wp >> 3;                            // 16 B chunks per row
+  // block ids of the keys [t_begin*32, t_end*32) into LDS (when they fit)
+  const int blk0 = t_begin * LM_KT / block_size;
+  const int nblk = (min(t_end * LM_KT, kmax) + block_size - 1) / block_size - blk0;
+  const bool tbl_ok = nblk <= 512;
+  if (tbl_ok)
+    for (int i = tid; i < nblk; i += 256) tbl[i] = table[blk0 + i];
+  __syncthreads();
+
+  // chunk c of a tile: key c / CH, columns (c % CH)*8 .. +8
+  auto fetch = [&](int t, int i) -> u16x8 {
+    const int c = tid + i * 256;
+    u16x8 v8 = {{0, 0, 0, 0, 0, 0, 0, 0}};
+    if (c < LM_KT * CH) {
+      const int kl = c / CH, col = (c - kl * CH) * 8;
+      const int key = t * LM_KT + kl;
       if (key < kmax && col < W) {
-        const long blk = table[key / block_size];
+        const int b = key / block_size;
+        const long blk = tbl_ok ? tbl[b - blk0] : table[b];
         v8 = *reinterpret_cast<const u16x8*>(
             cache + (blk * block_size + key % block_size) * (long)W + col);
       }
+    }
+    return v8;
+  };
+  auto put = [&](int i, const u16x8& v8) {
+    const int c = tid + i * 256;
+    if (c < LM_KT * CH) {
+      const int kl = c / CH, col = (c - kl * CH) * 8;
       *reinterpret_cast<u16x8*>(
           vt + (col >> 4) * 512 + ((kl >> 2) & 1) * 256 + (kl >> 3) * 64 +
           (kl & 3) * 16 + (col & 15)) = v8;
     }
+  };
+  u16x8 pre[PF ? NPF : 1];
+  if (PF && t_begin < t_end) {
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) pre[i] = fetch(t_begin, i);
+  }
+
+  for (int t = t_begin; t < t_end; ++t) {
+    const int k0 = t * LM_KT;
     __syncthreads();
+    // stage the whole (zero-padded) rows into the tr16 image: a 16 B chunk
+    // (8 columns of one key) stays contiguous, so the score MFMA reads its
+    // K fragments from the same image with ds_read_b128
+    if (PF) {
+#pragma unroll
+      for (int i = 0; i < NPF; ++i) put(i, pre[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < NPF; ++i) put(i, fetch(t, i));
+    }
+    __syncthreads();
+    if (PF && t + 1 < t_end) {          // next tile flies during the compute
+#pragma unroll
+      for (int i = 0; i < NPF; ++i) pre[i] = fetch(t + 1, i);
+    }
     if (!wave_on) continue;
     // ---- scores ------------------------------------------------------------
     float sc[8];
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
-      const int key = k0 + (n >> 2) * 8 + h2 * 4 + (n & 3);   // A row n
-      const bool kok = key < kmax;
-      const unsigned short* krow = cache;
-      if (kok) {
-        const long blk = table[key / block_size];
-        krow = cache + (blk * block_size + key % block_size) * (long)W;
-      }
+      // A row n is key k0 + (n>>2)*8 + h2*4 + (n&3); its image offset:
+      const unsigned short* krow = vt + h2 * 256 + (n >> 2) * 64 + (n & 3) * 16;
       f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kc = 0; kc < KQ; ++kc) {
         if (kc * 32 < Wp) {
           const int col = kc * 32 + g * 8;
-          bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-          const bf16x8 a = (kok && col < W) ? ld8(krow + col) : z;
+          const bf16x8 a = ld8(krow + (col >> 4) * 512 + (col & 15));
           sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kc], sacc, 0, 0,
                                                          0);
         }
@@ -193,8 +233,9 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     const unsigned vbase = (unsigned)(unsigned long long)(vt) +
                            (unsigned)(g * 128 + n * 8);
 #pragma unroll
-    for (int nb = 0; nb < NO / 4; ++nb) {
-      if (nb * 64 < rp && (!col_split || (nb & 3) == wv)) {
+    for (int lb = 0; lb < NBL; ++lb) {
+      const int nb = lb * CS + cpart;
+      if (nb * 64 < rp) {
         typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2;
         u32x2 tr[8];
         const unsigned va = vbase + (unsigned)(nb * 4096);
@@ -215,7 +256,7 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
             : "memory");
 #pragma unroll
         for (int nn = 0; nn < 4; ++nn) {
-          const int no = nb * 4 + nn;
+          const int no = lb * 4 + nn;
           bf16x8 a;
           unsigned* aw = reinterpret_cast<unsigned*>(&a);
           aw[0] = tr[2 * nn][0];
@@ -231,33 +272,22 @@ __global__ void __launch_bounds__(256) latent_attn_mfma_kernel(
     }
   }
   if (!wave_on || !row_ok) return;
-  // acc[no][rr] = O^T[col = no*16 + g*4 + rr][row n]
-  if (n_part == 1) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    float* orow = out + grow * r;
+  // acc[lb*4+nn][rr] = O^T[col = ((lb*CS+cpart)*4+nn)*16 + g*4 + rr][row n]
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  const long base = grow * n_part + blockIdx.y;
+  float* orow = (n_part == 1) ? out + grow * r : ws_acc + base * r;
+  const float mul = (n_part == 1) ? inv : 1.0f;
 #pragma unroll
-    for (int no = 0; no < NO; ++no)
+  for (int lb = 0; lb < NBL; ++lb)
 #pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r && (!col_split || ((no >> 2) & 3) == wv))
-          orow[col] = acc[no][rr] * inv;
-      }
-  } else {
-    // partials are indexed by the OUTPUT row: [row][part]
-    const long base = grow * n_part + blockIdx.y;
-    float* arow = ws_acc + base * r;
-#pragma unroll
-    for (int no = 0; no < NO; ++no)
+    for (int nn = 0; nn < 4; ++nn)
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
-        const int col = no * 16 + g * 4 + rr;
-        if (no * 16 < rp && col < r && (!col_split || ((no >> 2) & 3) == wv))
-          arow[col] = acc[no][rr];
+        const int col = ((lb * CS + cpart) * 4 + nn) * 16 + g * 4 + rr;
+        if (col < r) orow[col] = acc[lb * 4 + nn][rr] * mul;
       }
-    if (g == 0 && (!col_split || wv == 0)) {
-      ws_ml[base * 2] = m; ws_ml[base * 2 + 1] = l;
-    }
+  if (n_part > 1 && g == 0 && cpart == 0) {
+    ws_ml[base * 2] = m; ws_ml[base * 2 + 1] = l;
   }
 }
 
@@ -312,22 +342,34 @@ void launch_latent_attn_mfma(float* out, float* ws_acc, float* ws_ml,
   if (tokens == 0) return;
   const int cls = latent_attn_mfma_class(r + rd, r);
   const int rp = (r + 15) & ~15;
+  // decode with few heads: split the output columns over the waves
+  const int cs = (cu_q == nullptr) ? (heads <= 16 ? 4 : heads <= 32 ? 2 : 1)
+                                   : 1;
+  const int rows_wg = 64 / cs;
   int blocks;
   if (cu_q == nullptr)
-    blocks = n_seqs * ((heads + LM_ROWS - 1) / LM_ROWS);
+    blocks = n_seqs * ((heads + rows_wg - 1) / rows_wg);
   else
-    blocks = (int)(((long)tokens * heads + LM_ROWS - 1) / LM_ROWS) + n_seqs;
+    blocks = (int)(((long)tokens * heads + rows_wg - 1) / rows_wg) + n_seqs;
   dim3 grid(blocks, n_part);
-  // whole batches of four 16-column tiles (4096 B each)
-  const size_t lds = (size_t)((rp + 63) / 64) * 4096;
-#define LM_LAUNCH(KQ, NO)                                                    \
-  hipLaunchKernelGGL((latent_attn_mfma_kernel<KQ, NO>), grid, dim3(256), lds, \
-                     st, out, ws_acc, ws_ml, q, cache, block_tables, cu_q,   \
-                     seq_lens, n_seqs, heads, r, rd, block_size, table_width, \
-                     scale, n_part)
-  if (cls == 1) LM_LAUNCH(4, 8);
-  else if (cls == 2) LM_LAUNCH(10, 16);
-  else LM_LAUNCH(20, 32);
+  // whole batches of four 16-column tiles (4096 B each) over the padded row
+  const int Wp = (r + rd + 31) & ~31;
+  const size_t lds = (size_t)((Wp + 63) / 64) * 4096;
+#define LM_LAUNCH(KQ, NO, CS)                                                \
+  hipLaunchKernelGGL((latent_attn_mfma_kernel<KQ, NO, CS>), grid, dim3(256), \
+                     lds, st, out, ws_acc, ws_ml, q, cache, block_tables,    \
+                     cu_q, seq_lens, n_seqs, heads, r, rd, block_size,       \
+                     table_width, scale, n_part)
+#define LM_BY_CS(KQ, NO)                                                     \
+  do {                                                                       \
+    if (cs == 4) LM_LAUNCH(KQ, NO, 4);                                       \
+    else if (cs == 2) LM_LAUNCH(KQ, NO, 2);                                  \
+    else LM_LAUNCH(KQ, NO, 1);                                               \
+  } while (0)
+  if (cls == 1) LM_BY_CS(4, 8);
+  else if (cls == 2) LM_BY_CS(10, 16);
+  else LM_BY_CS(20, 32);
+#undef LM_BY_CS
 #undef LM_LAUNCH
   if (n_part > 1)
     hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tokens * heads),
