@@ -160,6 +160,60 @@ __global__ void __launch_bounds__(256) decay_attn_kernel(
   }
 }
 
+// Decode (one token per sequence): the step is a pure stream over the state,
+// so one workgroup takes a whole (sequence, head) state and moves it as
+// full rows: thread (rg, tc) owns columns 4*tc..4*tc+3 of rows rg, rg+RG, ...
+// (float4 per row; a wave covers whole 512 B rows at Dv = 128). Partial
+// outputs of the RG row groups are summed through LDS.
+template <typename T>
+__global__ void __launch_bounds__(256) decay_attn_decode_kernel(
+    float* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k,
+    const T* __restrict__ v, const float* __restrict__ decay,
+    float* __restrict__ state, const int* __restrict__ slots,
+    const int* __restrict__ ctx_lens, int heads, int D, int Dv, long q_stride,
+    long k_stride, long v_stride) {
+  extern __shared__ float smem[];
+  const int Dp = (D + 3) & ~3;      // keeps the float4 regions 16 B aligned
+  float* qs = smem;                 // [Dp]
+  float* ks = qs + Dp;              // [Dp]
+  float* vs = ks + Dp;              // [Dv]
+  float* part = vs + Dv;            // [RG][Dv]
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int TCn = Dv >> 2, RG = 256 / TCn;
+  const int rg = tid / TCn, tc = tid - rg * TCn;
+  for (int i = tid; i < D; i += 256) {
+    qs[i] = IO<T>::rnd(siluf_(IO<T>::ld(q + s * q_stride + h * D + i)));
+    ks[i] = IO<T>::rnd(siluf_(IO<T>::ld(k + s * k_stride + h * D + i)));
+  }
+  for (int i = tid; i < Dv; i += 256)
+    vs[i] = IO<T>::rnd(siluf_(IO<T>::ld(v + s * v_stride + h * Dv + i)));
+  __syncthreads();
+  const int slot = slots[s];
+  const bool load = slot >= 0 && ctx_lens[s] > 0;
+  const float a = decay[h];
+  float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (rg < RG) {
+    float* sp = state + (((long)max(slot, 0) * heads + h) * D) * (long)Dv + 4 * tc;
+    const float4 vv = *reinterpret_cast<const float4*>(vs + 4 * tc);
+    for (int i = rg; i < D; i += RG) {
+      float4 S = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (load) S = *reinterpret_cast<const float4*>(sp + (long)i * Dv);
+      const float ki = ks[i], qi = qs[i];
+      S.x = a * S.x + ki * vv.x; S.y = a * S.y + ki * vv.y;
+      S.z = a * S.z + ki * vv.z; S.w = a * S.w + ki * vv.w;
+      o.x += S.x * qi; o.y += S.y * qi; o.z += S.z * qi; o.w += S.w * qi;
+      if (slot >= 0) *reinterpret_cast<float4*>(sp + (long)i * Dv) = S;
+    }
+    *reinterpret_cast<float4*>(part + rg * Dv + 4 * tc) = o;
+  }
+  __syncthreads();
+  for (int c = tid; c < Dv; c += 256) {
+    float acc = 0.f;
+    for (int g2 = 0; g2 < RG; ++g2) acc += part[g2 * Dv + c];
+    out[((long)s * heads + h) * Dv + c] = acc;
+  }
+}
+
 // Sequential pass over a sequence's chunk states (one thread per state
 // element): ws[c] <- state before chunk c; the state after the last chunk
 // goes to the sequence's slot.
@@ -201,6 +255,16 @@ void launch_decay_attn(float* out, const T* q, const T* k, const T* v,
   if (n_seqs == 0) return;
   const size_t lds = (size_t)(2 * DA_TC * D + DA_TC * DA_VS) * sizeof(float);
   const int vz = (Dv + DA_VS - 1) / DA_VS;
+  if (cu_q == nullptr && Dv % 4 == 0 && Dv <= 1024) {
+    const int RG = 256 / (Dv / 4);
+    const size_t l2 = (size_t)(2 * ((D + 3) & ~3) + Dv + RG * Dv) * sizeof(float);
+    if (l2 <= 64 * 1024) {
+      hipLaunchKernelGGL((decay_attn_decode_kernel<T>), dim3(n_seqs, heads),
+                         dim3(256), l2, st, out, q, k, v, decay, state, slots,
+                         ctx_lens, heads, D, Dv, q_stride, k_stride, v_stride);
+      return;
+    }
+  }
   if (ws == nullptr || max_chunks <= 1) {
     hipLaunchKernelGGL((decay_attn_kernel<T>), dim3(n_seqs, heads, vz),
                        dim3(256), lds, st, out, q, k, v, decay, state, slots,
