@@ -135,7 +135,7 @@ class ModelRunner:
         # test_gpu_prefix_cache_and_chunked_prefill) while the full-length
         # serving shape (L == 1024 == bucket) runs and saves ~2.5 ms per
         # arrival. Until the padded-replay fault is isolated this stays
-        # off the default path — docs/TODO_ROUND3.md.
+        # off the default path — docs/TODO.md.
         if (ps.tp_size() == 1
                 and os.environ.get("XLLM_PREFILL_GRAPHS") == "1"):
             shared = os.environ.get("XLLM_PREFILL_GRAPH_SHARED_POOL") == "1"
