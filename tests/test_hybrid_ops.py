@@ -352,7 +352,9 @@ def test_norm_sigmoid_gate(dev):
 
 @pytest.mark.parametrize("dev", DEVS)
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("heads,r,rd", [(2, 40, 8), (19, 128, 32)])
+@pytest.mark.parametrize("heads,r,rd", [(2, 40, 8), (19, 128, 32),
+                                        (24, 512, 64), (40, 48, 8),
+                                        (70, 32, 0)])
 def test_latent_attn_decode_rows_of_unequal_context(dev, dt, heads, r, rd):
     """Decode rows whose contexts differ widely (the kernel may split long
     contexts over several workgroups and merge the parts)."""
