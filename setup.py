@@ -46,14 +46,17 @@ ext_modules = [
             "nvcc": HIP_FLAGS,
         },
     ),
-    # hybrid sequence mixers (latent attention, decayed linear attention),
-    # grouped norms and routed experts; bf16 and fp32 activations
+    # hybrid sequence mixers (latent attention, decayed and gated linear
+    # recurrences, soft-capped paged attention, short convolutions), grouped
+    # norms, residual streams and routed experts; bf16 and fp32 activations
     CUDAExtension(
         name="xllm_service_amd._ops_hybrid",
         sources=[
             os.path.join(HYB, f)
             for f in ("bindings.cpp", "norms.hip", "latent_attn.hip",
-                      "latent_attn_mfma.hip", "decay_attn.hip", "moe.hip")
+                      "latent_attn_mfma.hip", "decay_attn.hip", "moe.hip",
+                      "streams.hip", "short_conv.hip",
+                      "gated_recurrence.hip", "capped_attn.hip")
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],

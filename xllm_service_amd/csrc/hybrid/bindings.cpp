@@ -49,6 +49,38 @@ void launch_moe_route(int*, float*, const float*, int, int, int, int, int,
 template <typename T>
 void launch_moe_combine(float*, const T*, const int*, const float*, long, int,
                         int, hipStream_t);
+template <typename TO>
+void launch_streams_mix_norm(TO*, const float*, const float*, const float*,
+                             const float*, float, int, int, int, hipStream_t);
+template <typename T>
+void launch_streams_update(float*, const float*, const float*, const T*, float,
+                           const T*, float, long, int, int, hipStream_t);
+template <typename T>
+void launch_relu_sq(T*, long, hipStream_t);
+template <typename T>
+void launch_softcap(float*, const T*, float, long, hipStream_t);
+template <typename T>
+void launch_short_conv(T*, long, T*, const long*, int, const T*, long,
+                       const T*, const T*, const T*, long, int, const int*,
+                       const int*, const int*, int, int, int, int, int, int,
+                       int, const long*, const double*, hipStream_t);
+template <typename T>
+void launch_short_conv_state(T*, long, const T*, long, const int*, const int*,
+                             int, int, int, hipStream_t);
+template <typename T>
+void launch_gated_recurrence(int, float*, const T*, const T*, const T*,
+                             const T*, long, long, long, long, const float*,
+                             const float*, const float*, float, float, float*,
+                             const int*, const int*, const int*, int, int, int,
+                             int, int, int, int, float*, float*, hipStream_t);
+template <typename T>
+void launch_gated_group_norm(T*, const float*, const float*, int, const T*,
+                             long, float, int, int, int, int, int,
+                             hipStream_t);
+template <typename T>
+void launch_capped_attn(float*, const T*, const T*, const T*, const int*,
+                        const int*, const int*, int, int, int, int, int, int,
+                        int, int, float, float, long, hipStream_t);
 }  // namespace hyb
 }  // namespace xllm
 
@@ -332,6 +364,294 @@ void moe_combine(Tensor out, Tensor y, Tensor rows, Tensor wts) {
     hy::launch_moe_combine<bf>(ptr<float>(out), ptr<bf>(y), ptr<int>(rows), ptr<float>(wts), T, width, top, cur());
 }
 
+// x fp32 [T, S, W]; out [T, W] = layernorm(sum_s w_in[s] x[:, s]) * g + b
+void streams_mix_norm(Tensor out, Tensor x, c10::optional<Tensor> w_in,
+                      Tensor g, Tensor b, double eps) {
+  CHK_ACT(out); CHK_F32C(x); CHK_F32C(g); CHK_F32C(b);
+  TORCH_CHECK(x.dim() == 3 && out.dim() == 2 && out.is_contiguous());
+  const int T = x.size(0), S = x.size(1), W = x.size(2);
+  TORCH_CHECK(out.size(0) == T && out.size(1) == W && g.numel() == W &&
+              b.numel() == W && S >= 1 && S <= 8, "streams: bad shapes");
+  TORCH_CHECK((size_t)W * 4 <= 60 * 1024, "width too large for LDS");
+  const float* wi = nullptr;
+  if (w_in.has_value()) {
+    CHK_F32C(*w_in);
+    TORCH_CHECK(w_in->numel() == S);
+    wi = ptr<float>(*w_in);
+  }
+  if (is_f32(out))
+    hy::launch_streams_mix_norm<float>(ptr<float>(out), ptr<float>(x), wi, ptr<float>(g), ptr<float>(b), eps, T, S, W, cur());
+  else
+    hy::launch_streams_mix_norm<bf>(ptr<bf>(out), ptr<float>(x), wi, ptr<float>(g), ptr<float>(b), eps, T, S, W, cur());
+}
+
+// x[:, j] <- sum_s mix[s, j] x[:, s] + w_out[j] (a1 y1 + a2 y2), in place
+void streams_update(Tensor x, c10::optional<Tensor> mix,
+                    c10::optional<Tensor> w_out, Tensor y1, double a1,
+                    c10::optional<Tensor> y2, double a2) {
+  CHK_F32C(x); CHK_ACT(y1);
+  TORCH_CHECK(x.dim() == 3 && y1.is_contiguous());
+  const long T = x.size(0);
+  const int S = x.size(1), W = x.size(2);
+  TORCH_CHECK(S >= 1 && S <= 8 && y1.numel() == T * W);
+  const float *mp = nullptr, *op = nullptr;
+  if (mix.has_value()) {
+    CHK_F32C(*mix);
+    TORCH_CHECK(mix->numel() == S * S);
+    mp = ptr<float>(*mix);
+  }
+  if (w_out.has_value()) {
+    CHK_F32C(*w_out);
+    TORCH_CHECK(w_out->numel() == S);
+    op = ptr<float>(*w_out);
+  }
+  const void* y2p = nullptr;
+  if (y2.has_value()) {
+    CHK_ACT(*y2);
+    TORCH_CHECK(y2->is_contiguous() && y2->numel() == T * W &&
+                y2->dtype() == y1.dtype());
+    y2p = y2->data_ptr();
+  }
+  if (is_f32(y1))
+    hy::launch_streams_update<float>(ptr<float>(x), mp, op, ptr<float>(y1), a1, (const float*)y2p, a2, T, S, W, cur());
+  else
+    hy::launch_streams_update<bf>(ptr<float>(x), mp, op, ptr<bf>(y1), a1, (const bf*)y2p, a2, T, S, W, cur());
+}
+
+void relu_sq(Tensor x) {
+  CHK_ACT(x);
+  TORCH_CHECK(x.is_contiguous());
+  if (is_f32(x)) hy::launch_relu_sq<float>(ptr<float>(x), x.numel(), cur());
+  else hy::launch_relu_sq<bf>(ptr<bf>(x), x.numel(), cur());
+}
+
+void softcap(Tensor out, Tensor x, double cap) {
+  CHK_F32C(out); CHK_ACT(x);
+  TORCH_CHECK(x.is_contiguous() && out.numel() == x.numel() && cap > 0);
+  if (is_f32(x)) hy::launch_softcap<float>(ptr<float>(out), ptr<float>(x), cap, x.numel(), cur());
+  else hy::launch_softcap<bf>(ptr<float>(out), ptr<bf>(x), cap, x.numel(), cur());
+}
+
+// Short causal convolution of x [T, heads*hd] (row view) with per-channel
+// filters w [heads*hd, taps]; the sequence's earlier inputs come from
+// state[slot, :, state_off : state_off + heads*hd]. Result to `out` (row
+// view) or into the paged `cache` [blocks, heads, block, hd] at slot_mapping.
+void short_conv(c10::optional<Tensor> out, c10::optional<Tensor> cache,
+                c10::optional<Tensor> slot_mapping, Tensor x, Tensor w,
+                c10::optional<Tensor> bias, Tensor state, long state_off,
+                Tensor slots, c10::optional<Tensor> cu_q, Tensor ctx_lens,
+                long heads, long hd, bool act_silu, long rot_dims,
+                c10::optional<Tensor> pos, c10::optional<Tensor> inv_freq) {
+  CHK_ACT(x); CHK_ACT(w); CHK_ACT(state); CHK_I32C(slots); CHK_I32C(ctx_lens);
+  TORCH_CHECK(x.dim() == 2 && w.dim() == 2 && w.is_contiguous() &&
+              state.dim() == 3 && state.is_contiguous() &&
+              w.dtype() == x.dtype() && state.dtype() == x.dtype());
+  const int T = x.size(0), C = heads * hd, taps = w.size(1);
+  TORCH_CHECK(x.size(1) == C && w.size(0) == C && taps >= 1 && taps <= 16 &&
+              state.size(1) == taps - 1 && state_off >= 0 &&
+              state_off + C <= state.size(2), "short_conv: bad shapes");
+  const int n_seqs = slots.numel();
+  TORCH_CHECK(ctx_lens.numel() == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  const void* bp = nullptr;
+  if (bias.has_value()) {
+    CHK_ACT(*bias);
+    TORCH_CHECK(bias->numel() == C && bias->is_contiguous() &&
+                bias->dtype() == x.dtype());
+    bp = bias->data_ptr();
+  }
+  const long* posp = nullptr;
+  const double* fp = nullptr;
+  if (rot_dims > 0) {
+    TORCH_CHECK(pos.has_value() && inv_freq.has_value() && rot_dims % 2 == 0 &&
+                rot_dims <= hd);
+    CHK_I64C(*pos);
+    TORCH_CHECK(pos->numel() == T && inv_freq->is_cuda() &&
+                inv_freq->dtype() == torch::kDouble &&
+                inv_freq->is_contiguous() &&
+                inv_freq->numel() == rot_dims / 2);
+    posp = ptr<long>(*pos);
+    fp = ptr<double>(*inv_freq);
+  }
+  void* outp = nullptr;
+  long out_stride = 0;
+  void* cachep = nullptr;
+  const long* smp = nullptr;
+  int bs = 1;
+  if (cache.has_value()) {
+    CHK_ACT(*cache);
+    TORCH_CHECK(slot_mapping.has_value());
+    CHK_I64C(*slot_mapping);
+    TORCH_CHECK(cache->dim() == 4 && cache->is_contiguous() &&
+                cache->size(1) == heads && cache->size(3) == hd &&
+                cache->dtype() == x.dtype() && slot_mapping->numel() == T);
+    cachep = cache->data_ptr();
+    smp = ptr<long>(*slot_mapping);
+    bs = cache->size(2);
+  } else {
+    TORCH_CHECK(out.has_value());
+    CHK_ACT(*out);
+    TORCH_CHECK(out->dim() == 2 && out->size(0) == T && out->size(1) == C &&
+                out->dtype() == x.dtype());
+    outp = out->data_ptr();
+    out_stride = out->stride(0);
+  }
+  if (is_f32(x))
+    hy::launch_short_conv<float>((float*)outp, out_stride, (float*)cachep, smp, bs, ptr<float>(x), x.stride(0), ptr<float>(w), (const float*)bp, ptr<float>(state), state.size(2), state_off, ptr<int>(slots), cu, ptr<int>(ctx_lens), T, n_seqs, heads, hd, taps, act_silu, rot_dims, posp, fp, cur());
+  else
+    hy::launch_short_conv<bf>((bf*)outp, out_stride, (bf*)cachep, smp, bs, ptr<bf>(x), x.stride(0), ptr<bf>(w), (const bf*)bp, ptr<bf>(state), state.size(2), state_off, ptr<int>(slots), cu, ptr<int>(ctx_lens), T, n_seqs, heads, hd, taps, act_silu, rot_dims, posp, fp, cur());
+}
+
+// state [slots, taps-1, C] <- the last taps-1 inputs after this step's rows
+void short_conv_state(Tensor state, Tensor x, Tensor slots,
+                      c10::optional<Tensor> cu_q) {
+  CHK_ACT(state); CHK_ACT(x); CHK_I32C(slots);
+  TORCH_CHECK(state.dim() == 3 && state.is_contiguous() && x.dim() == 2 &&
+              x.size(1) == state.size(2) && x.dtype() == state.dtype());
+  const int n_seqs = slots.numel(), taps = state.size(1) + 1;
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == x.size(0), "decode: one sequence per token");
+  }
+  if (is_f32(x))
+    hy::launch_short_conv_state<float>(ptr<float>(state), state.size(2), ptr<float>(x), x.stride(0), ptr<int>(slots), cu, n_seqs, x.size(1), taps, cur());
+  else
+    hy::launch_short_conv_state<bf>(ptr<bf>(state), state.size(2), ptr<bf>(x), x.stride(0), ptr<int>(slots), cu, n_seqs, x.size(1), taps, cur());
+}
+
+// kind 0: selective state space (q = C, k = B shared per group, v = x,
+//   g = dt_raw [T, H]; p0 = dt_bias, p1 = A_log, p2 = D skip)
+// kind 1: gated linear attention (g = z [T, H*D]; p0 = z bias [H*D];
+//   c0 = 1/tau, c1 = query scale)
+// out fp32 [T, H, Dv]; state fp32 [slots, H, D, Dv]; q/k [T, groups*D] views
+void gated_recurrence(long kind, Tensor out, Tensor q, Tensor k, Tensor v,
+                      Tensor g, Tensor p0, c10::optional<Tensor> p1,
+                      c10::optional<Tensor> p2, double c0, double c1,
+                      Tensor state, Tensor slots, c10::optional<Tensor> cu_q,
+                      Tensor ctx_lens, long groups, long max_q_len) {
+  CHK_F32C(out); CHK_ACT(q); CHK_ACT(k); CHK_ACT(v); CHK_ACT(g); CHK_F32C(p0);
+  CHK_F32C(state); CHK_I32C(slots); CHK_I32C(ctx_lens);
+  TORCH_CHECK(state.dim() == 4 && q.dim() == 2 && k.dim() == 2 &&
+              v.dim() == 2 && g.dim() == 2 && q.dtype() == k.dtype() &&
+              q.dtype() == v.dtype() && q.dtype() == g.dtype());
+  const int H = state.size(1), D = state.size(2), Dv = state.size(3);
+  const int T = q.size(0);
+  TORCH_CHECK(kind == 0 || kind == 1);
+  TORCH_CHECK(groups >= 1 && H % groups == 0 && q.size(1) == groups * D &&
+              k.size(1) == groups * D && v.size(1) == H * Dv &&
+              k.size(0) == T && v.size(0) == T && g.size(0) == T,
+              "gated_recurrence: bad shapes");
+  TORCH_CHECK(D <= 256, "key dim > 256 unsupported");
+  TORCH_CHECK(out.numel() == (long)T * H * Dv);
+  const float *p1p = nullptr, *p2p = nullptr;
+  if (kind == 0) {
+    TORCH_CHECK(g.size(1) == H && p0.numel() == H && p1.has_value());
+    CHK_F32C(*p1);
+    TORCH_CHECK(p1->numel() == H);
+    p1p = ptr<float>(*p1);
+    if (p2.has_value()) {
+      CHK_F32C(*p2);
+      TORCH_CHECK(p2->numel() == H);
+      p2p = ptr<float>(*p2);
+    }
+  } else {
+    TORCH_CHECK(groups == H && g.size(1) == H * D && p0.numel() == H * D);
+  }
+  const int n_seqs = slots.numel();
+  TORCH_CHECK(ctx_lens.numel() == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  int chunk = 128, max_chunks = 1;
+  Tensor ws, wa;
+  if (cu != nullptr) {
+    const long bound = max_q_len > 0 ? std::min<long>(max_q_len, T) : T;
+    const long per_seq = (long)H * D * Dv * 4;
+    while ((bound + chunk - 1) / chunk * n_seqs * per_seq > (1L << 31))
+      chunk *= 2;                             // keep the scratch under 2 GiB
+    if (bound >= 2L * chunk) {
+      max_chunks = (int)((bound + chunk - 1) / chunk);
+      ws = torch::empty({(long)n_seqs * max_chunks, (long)H, (long)D, (long)Dv},
+                        state.options());
+      wa = torch::empty({(long)n_seqs * max_chunks, (long)H,
+                         (long)(kind == 0 ? 1 : D)}, state.options());
+    }
+  }
+  float* wsp = max_chunks > 1 ? ptr<float>(ws) : nullptr;
+  float* wap = max_chunks > 1 ? ptr<float>(wa) : nullptr;
+  if (is_f32(q))
+    hy::launch_gated_recurrence<float>(kind, ptr<float>(out), ptr<float>(q), ptr<float>(k), ptr<float>(v), ptr<float>(g), q.stride(0), k.stride(0), v.stride(0), g.stride(0), ptr<float>(p0), p1p, p2p, c0, c1, ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, chunk, max_chunks, wsp, wap, cur());
+  else
+    hy::launch_gated_recurrence<bf>(kind, ptr<float>(out), ptr<bf>(q), ptr<bf>(k), ptr<bf>(v), ptr<bf>(g), q.stride(0), k.stride(0), v.stride(0), g.stride(0), ptr<float>(p0), p1p, p2p, c0, c1, ptr<float>(state), ptr<int>(slots), cu, ptr<int>(ctx_lens), n_seqs, H, groups, D, Dv, chunk, max_chunks, wsp, wap, cur());
+}
+
+// out [rows, n] from o fp32 [rows, n], gate [rows, n] (row view), w fp32 with
+// n or n/groups entries
+void gated_group_norm(Tensor out, Tensor o, Tensor w, Tensor gate, double eps,
+                      long groups, bool act_silu, bool gate_first) {
+  CHK_ACT(out); CHK_F32C(o); CHK_F32C(w); CHK_ACT(gate);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && gate.dim() == 2);
+  const int rows = out.size(0), n = out.size(1);
+  TORCH_CHECK(o.numel() == (long)rows * n && gate.size(0) == rows &&
+              gate.size(1) == n && gate.dtype() == out.dtype() &&
+              groups >= 1 && n % groups == 0 &&
+              (w.numel() == n || w.numel() == n / groups));
+  if (is_f32(out))
+    hy::launch_gated_group_norm<float>(ptr<float>(out), ptr<float>(o), ptr<float>(w), w.numel(), ptr<float>(gate), gate.stride(0), eps, rows, n, groups, act_silu, gate_first, cur());
+  else
+    hy::launch_gated_group_norm<bf>(ptr<bf>(out), ptr<float>(o), ptr<float>(w), w.numel(), ptr<bf>(gate), gate.stride(0), eps, rows, n, groups, act_silu, gate_first, cur());
+}
+
+// out fp32 [T, H, Dv]; q [T, H*D] row view; caches [blocks, n_kv, bs, D|Dv]
+void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                 Tensor block_tables, c10::optional<Tensor> cu_q,
+                 Tensor seq_lens, long heads, double scale, double cap) {
+  CHK_F32C(out); CHK_ACT(q); CHK_ACT(k_cache); CHK_ACT(v_cache);
+  CHK_I32C(block_tables); CHK_I32C(seq_lens);
+  TORCH_CHECK(q.dim() == 2 && k_cache.dim() == 4 && v_cache.dim() == 4 &&
+              k_cache.is_contiguous() && v_cache.is_contiguous() &&
+              q.dtype() == k_cache.dtype() && q.dtype() == v_cache.dtype() &&
+              block_tables.dim() == 2);
+  const int T = q.size(0), n_kv = k_cache.size(1), bs = k_cache.size(2);
+  const int D = k_cache.size(3), Dv = v_cache.size(3);
+  TORCH_CHECK(q.size(1) == heads * D && heads % n_kv == 0 &&
+              v_cache.size(1) == n_kv && v_cache.size(2) == bs &&
+              v_cache.size(0) == k_cache.size(0) && Dv <= 64 * 8,
+              "capped_attn: bad shapes");
+  TORCH_CHECK(out.numel() == (long)T * heads * Dv);
+  const int n_seqs = seq_lens.numel();
+  TORCH_CHECK(block_tables.size(0) == n_seqs);
+  const int* cu = nullptr;
+  if (cu_q.has_value()) {
+    CHK_I32C(*cu_q);
+    TORCH_CHECK(cu_q->numel() == n_seqs + 1);
+    cu = ptr<int>(*cu_q);
+  } else {
+    TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  TORCH_CHECK((size_t)4 * D * 4 <= 64 * 1024, "query row too wide for LDS");
+  if (is_f32(q))
+    hy::launch_capped_attn<float>(ptr<float>(out), ptr<float>(q), ptr<float>(k_cache), ptr<float>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), cur());
+  else
+    hy::launch_capped_attn<bf>(ptr<float>(out), ptr<bf>(q), ptr<bf>(k_cache), ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T, n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap, q.stride(0), cur());
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -345,4 +665,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("decay_attn", &decay_attn);
   m.def("moe_route", &moe_route);
   m.def("moe_combine", &moe_combine);
+  m.def("streams_mix_norm", &streams_mix_norm);
+  m.def("streams_update", &streams_update);
+  m.def("relu_sq", &relu_sq);
+  m.def("softcap", &softcap);
+  m.def("short_conv", &short_conv);
+  m.def("short_conv_state", &short_conv_state);
+  m.def("gated_recurrence", &gated_recurrence);
+  m.def("gated_group_norm", &gated_group_norm);
+  m.def("capped_attn", &capped_attn);
 }

@@ -90,6 +90,47 @@ __global__ void norm_sigmoid_gate_kernel(T* __restrict__ out,
   }
 }
 
+// Gate and grouped RMS norm of an fp32 row, in either order:
+//   gate_first: z = o * act(gate);  out = z / rms_g(z) * w
+//   else:       out = o / rms_g(o) * w * act(gate)
+// act = silu or sigmoid; rms over `groups` equal consecutive parts; w has
+// w_period entries and repeats (w_period = n: one weight per column;
+// w_period = n / groups: the same weights for every group).
+template <typename T>
+__global__ void gated_group_norm_kernel(
+    T* __restrict__ out, const float* __restrict__ o,
+    const float* __restrict__ w, int w_period, const T* __restrict__ gate,
+    long gate_stride, float eps, int n, int groups, int act_silu,
+    int gate_first) {
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int nw = blockDim.x >> 6;
+  const int gs = n / groups;
+  const float* orow = o + (long)row * n;
+  const T* gr = gate + (long)row * gate_stride;
+  T* dst = out + (long)row * n;
+  for (int g = wid; g < groups; g += nw) {
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += 64) {
+      const int c = g * gs + i;
+      float z = orow[c];
+      if (gate_first) {
+        const float gv = IO<T>::ld(gr + c);
+        z *= act_silu ? siluf_(gv) : sigmoidf_(gv);
+      }
+      ss += z * z;
+    }
+    ss = wave_reduce_sum(ss);
+    const float rs = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int i = lane; i < gs; i += 64) {
+      const int c = g * gs + i;
+      const float gv = IO<T>::ld(gr + c);
+      const float a = act_silu ? siluf_(gv) : sigmoidf_(gv);
+      IO<T>::st(dst + c, orow[c] * a * rs * w[c % w_period]);
+    }
+  }
+}
+
 // out[r, i] = silu(x[r, i]) * x[r, F + i]
 template <typename T>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ x,
@@ -160,6 +201,16 @@ void launch_norm_sigmoid_gate(T* out, const float* o, const float* w,
                      st, out, o, w, gate, eps, n, gate_stride);
 }
 template <typename T>
+void launch_gated_group_norm(T* out, const float* o, const float* w,
+                             int w_period, const T* gate, long gate_stride,
+                             float eps, int rows, int n, int groups,
+                             int act_silu, int gate_first, hipStream_t st) {
+  if (rows == 0) return;
+  hipLaunchKernelGGL((gated_group_norm_kernel<T>), dim3(rows), dim3(256), 0,
+                     st, out, o, w, w_period, gate, gate_stride, eps, n,
+                     groups, act_silu, gate_first);
+}
+template <typename T>
 void launch_silu_mul(T* out, const T* x, long rows, int F, hipStream_t st) {
   const long n = rows * (long)F;
   if (n == 0) return;
@@ -185,6 +236,9 @@ void launch_rope_interleaved(T* x, const long* pos, const double* inv_freq,
                                             const T*, float, int, int, long,  \
                                             hipStream_t);                     \
   template void launch_silu_mul<T>(T*, const T*, long, int, hipStream_t);     \
+  template void launch_gated_group_norm<T>(T*, const float*, const float*,    \
+                                           int, const T*, long, float, int,   \
+                                           int, int, int, int, hipStream_t);  \
   template void launch_rope_interleaved<T>(T*, const long*, const double*,    \
                                            float, int, int, int, long, long,  \
                                            int, hipStream_t);

@@ -13,8 +13,9 @@ import torch
 from xllm_service_amd import ops
 from xllm_service_amd.models.config import ModelConfig
 
-from .cache_spec import (PagedKV, PagedLatent, RecurrentState, SharedCache,
-                         default_specs, needs_state_slots)
+from .cache_spec import (CacheGroup, ConvState, PagedKV, PagedLatent,
+                         RecurrentState, SharedCache, default_specs,
+                         flat_specs, needs_state_slots)
 from .metadata import AttnMetadata
 from .scheduler import StepPlan
 from .sequence import Sequence
@@ -40,24 +41,31 @@ class ModelRunner:
         # one entry per layer, shaped by its spec (engine/cache_spec.py)
         self.kv_caches: List = []
         for spec in self.specs:
-            if isinstance(spec, PagedKV):
-                self.kv_caches.append(tuple(
-                    torch.zeros(num_blocks, spec.n_kv, BLOCK_SIZE,
-                                spec.head_dim, dtype=dtype, device=device)
-                    for _ in range(2)))
-            elif isinstance(spec, PagedLatent):
-                self.kv_caches.append(torch.zeros(
-                    num_blocks, BLOCK_SIZE, spec.width, dtype=dtype,
-                    device=device))
-            elif isinstance(spec, RecurrentState):
-                self.kv_caches.append(torch.zeros(
-                    max(num_state_slots, 1), spec.heads, spec.dim, spec.vdim,
-                    dtype=torch.float32, device=device))
-            elif isinstance(spec, SharedCache):
-                self.kv_caches.append(self.kv_caches[spec.source])
-            else:
-                raise TypeError(f"unknown cache spec {spec!r}")
+            self.kv_caches.append(self._allocate(spec))
         self.cpu_kv_caches: List[Tuple[torch.Tensor, torch.Tensor]] = []
+
+    def _allocate(self, spec):
+        dtype, device = self.dtype, self.device
+        slots = max(self.num_state_slots, 1)
+        if isinstance(spec, PagedKV):
+            return tuple(
+                torch.zeros(self.num_blocks, spec.n_kv, BLOCK_SIZE, d,
+                            dtype=dtype, device=device)
+                for d in (spec.head_dim, spec.value_dim))
+        if isinstance(spec, PagedLatent):
+            return torch.zeros(self.num_blocks, BLOCK_SIZE, spec.width,
+                               dtype=dtype, device=device)
+        if isinstance(spec, RecurrentState):
+            return torch.zeros(slots, spec.heads, spec.dim, spec.vdim,
+                               dtype=torch.float32, device=device)
+        if isinstance(spec, ConvState):
+            return torch.zeros(slots, max(spec.taps - 1, 0), spec.channels,
+                               dtype=dtype, device=device)
+        if isinstance(spec, CacheGroup):
+            return tuple(self._allocate(p) for p in spec.parts)
+        if isinstance(spec, SharedCache):
+            return self.kv_caches[spec.source]
+        raise TypeError(f"unknown cache spec {spec!r}")
 
     @staticmethod
     def specs_for(model, cfg: ModelConfig):
@@ -74,11 +82,17 @@ class ModelRunner:
     def paged_tensors(self) -> List[torch.Tensor]:
         """Every block-addressed cache tensor, each once (migration/export)."""
         out = []
-        for spec, c in zip(self.specs, self.kv_caches):
+
+        def walk(spec, c):
             if isinstance(spec, PagedKV):
                 out.extend(c)
             elif isinstance(spec, PagedLatent):
                 out.append(c)
+            elif isinstance(spec, CacheGroup):
+                for p, t in zip(spec.parts, c):
+                    walk(p, t)
+        for spec, c in zip(self.specs, self.kv_caches):
+            walk(spec, c)
         return out
 
     def alloc_cpu_caches(self, num_cpu_blocks: int):
@@ -110,7 +124,8 @@ class ModelRunner:
         if specs is None:
             specs = default_specs(cfg, n_kv_local)
         budget -= num_state_slots * sum(
-            s.slot_bytes() for s in specs if isinstance(s, RecurrentState))
+            s.slot_bytes() for s in flat_specs(specs)
+            if isinstance(s, (RecurrentState, ConvState)))
         per_block = max(sum(s.block_bytes(BLOCK_SIZE, dtype_bytes)
                             for s in specs), 1)
         n = max(budget // per_block, 16)

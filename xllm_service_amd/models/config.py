@@ -10,7 +10,7 @@ from typing import List, Optional
 @dataclass
 class ModelConfig:
     name: str = "llama"
-    architecture: str = "llama"          # llama | opt | qwen2 | qwen2_vl | pugovik
+    architecture: str = "llama"   # llama | opt | qwen2 | qwen2_vl | pugovik | dunusun
     vocab_size: int = 128256
     hidden_size: int = 4096
     intermediate_size: int = 14336
@@ -155,6 +155,64 @@ def pugovik_from_dict(d: dict, name: str = "pugovik",
         max_position=1 << 20, layers=layers, model_dir=model_dir)
 
 
+@dataclass
+class DunusunConfig(ModelConfig):
+    """Dunusun: layers of a selective state space mixer (`mamba2`) or of a
+    soft-capped softmax attention beside a gated linear attention
+    (`parallel`), dense squared-ReLU feed-forwards, layer norms with bias,
+    several residual streams mixed around every sublayer, a run of layers
+    that repeats with the same weights, soft-capped logits."""
+    layers: List[HybridLayerConfig] = field(default_factory=list)
+    streams: Optional[int] = None       # None: one plain residual
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 1
+    logit_softcap: Optional[float] = None
+    model_dir: Optional[str] = None     # weights live here (None = random)
+
+    @property
+    def layer_runs(self) -> List[int]:
+        """Layer index of every layer run, in execution order (a looped
+        layer appears once per pass; each run owns its cache and state)."""
+        n = len(self.layers)
+        body = list(range(self.loop_start, self.loop_stop))
+        return (list(range(self.loop_start)) + body * self.loop_times
+                + list(range(self.loop_stop, n)))
+
+    @property
+    def has_recurrent_state(self) -> bool:
+        return True
+
+
+def dunusun_from_dict(d: dict, name: str = "dunusun",
+                      model_dir: Optional[str] = None) -> DunusunConfig:
+    layers = [HybridLayerConfig(type=l["type"], mixer=dict(l["mixer"]),
+                                mlp=l.get("mlp"))
+              for l in d["layers"]]
+    for i, l in enumerate(layers):
+        if l.type not in ("mamba2", "parallel"):
+            raise ValueError(f"layer {i}: unknown mixer type {l.type!r}")
+        if l.mlp is not None and l.mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind")
+    lp = d.get("loop") or {}
+    start, stop = int(lp.get("start", 0)), int(lp.get("stop", 0))
+    times = int(lp.get("times", 1))
+    if not lp:
+        start = stop = 0
+        times = 1
+    if not (0 <= start <= stop <= len(layers)) or times < 0:
+        raise ValueError("loop: need 0 <= start <= stop <= layers")
+    streams = d.get("streams")
+    cap = d.get("logit_softcap")
+    return DunusunConfig(
+        name=name, architecture="dunusun", vocab_size=int(d["vocab"]),
+        hidden_size=int(d["width"]), num_layers=len(layers),
+        rms_eps=float(d["norm"]["eps"]), max_position=1 << 20, layers=layers,
+        streams=None if streams is None else int(streams),
+        loop_start=start, loop_stop=stop, loop_times=times,
+        logit_softcap=float(cap) if cap else None, model_dir=model_dir)
+
+
 def load_model_dir(path: str) -> ModelConfig:
     """Read <path>/config.json and pick the config class by its
     `architecture` field."""
@@ -164,6 +222,9 @@ def load_model_dir(path: str) -> ModelConfig:
     if arch == "pugovik":
         return pugovik_from_dict(d, name=os.path.basename(
             os.path.normpath(path)) or "pugovik", model_dir=path)
+    if arch == "dunusun":
+        return dunusun_from_dict(d, name=os.path.basename(
+            os.path.normpath(path)) or "dunusun", model_dir=path)
     raise ValueError(f"{path}: unsupported architecture "
                      f"{d.get('architecture')!r}")
 

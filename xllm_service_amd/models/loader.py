@@ -49,6 +49,22 @@ def iter_safetensors(path: str) -> Iterator[Tuple[str, torch.Tensor]]:
             mm.close()
 
 
+def safetensors_shapes(path: str) -> Dict[str, Tuple[int, ...]]:
+    """{name: shape} of every tensor in a model folder, from the file
+    headers alone."""
+    out: Dict[str, Tuple[int, ...]] = {}
+    for fn in sorted(os.listdir(path)):
+        if not fn.endswith(".safetensors"):
+            continue
+        with open(os.path.join(path, fn), "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(n))
+        for name, info in header.items():
+            if name != "__metadata__":
+                out[name] = tuple(info["shape"])
+    return out
+
+
 def load_model_dir_tensors(path: str) -> Dict[str, torch.Tensor]:
     """All tensors of every *.safetensors file in a model folder."""
     out: Dict[str, torch.Tensor] = {}

@@ -9,7 +9,21 @@ LatentAttention        softmax attention whose keys and values are linear
 DecayLinearAttention   per-head state S <- decay * S + k v^T, o = S^T q with
                        SiLU feature maps; the state lives in a slot pool.
 
-Both take the slice of a merged input projection that belongs to them and
+SelectiveStateSpace    Mamba-2 style mixer: short convolution + SiLU on
+                       [x | B | C], per-head scalar decay exp(-exp(A) dt),
+                       state S <- a S + dt B x^T, y = S^T C + D x, SiLU gate,
+                       grouped RMS norm.
+CappedAttention        softmax attention with grouped key/value heads, a
+                       short convolution on q/k/v, rotary pairs on part of
+                       each head, a tanh soft cap on the scores, separate
+                       key and value widths, sigmoid output gate.
+GatedLinearAttention   S <- diag(alpha) S + k v^T, o = S^T q with a low-rank
+                       per-channel decay alpha = sigmoid(.)^(1/tau); RMS norm
+                       per head, SiLU gate.
+ParallelMixer          two mixers reading the same input, outputs added
+                       with fixed weights.
+
+All take the slice of a merged input projection that belongs to them and
 return the mixer output in the model dtype. Sizes and constants are
 constructor arguments.
 """
@@ -22,8 +36,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from xllm_service_amd.engine.cache_spec import (PagedLatent, RecurrentState,
-                                                SharedCache)
+from xllm_service_amd.engine.cache_spec import (CacheGroup, ConvState,
+                                                PagedKV, PagedLatent,
+                                                RecurrentState, SharedCache)
 from xllm_service_amd.engine.metadata import AttnMetadata
 from xllm_service_amd.ops import hybrid as hops
 
@@ -162,3 +177,201 @@ class DecayLinearAttention(nn.Module):
         y = hops.norm_sigmoid_gate(o.view(T, b), self.out_norm, gate,
                                    self.eps, proj.dtype)
         return F.linear(y, self.o_proj)
+
+
+def _halves(meta: AttnMetadata, aux):
+    """The prefill and the decode part of a batch as (rows, cu_q, ctx_lens,
+    state_slots, seq_lens, block_tables, max_len) tuples."""
+    np_, nd = meta.num_prefill_tokens, meta.num_decode_tokens
+    out = []
+    if np_:
+        out.append((slice(0, np_), meta.cu_q, meta.prefill_ctx_lens,
+                    meta.prefill_state_slots, meta.prefill_seq_lens,
+                    meta.prefill_block_tables, meta.max_prefill_len))
+    if nd:
+        out.append((slice(np_, np_ + nd), None, aux["decode_ctx_lens"],
+                    meta.decode_state_slots, meta.decode_seq_lens,
+                    meta.decode_block_tables, 1))
+    return out
+
+
+class SelectiveStateSpace(nn.Module):
+    """in_proj rows: [z: inner | x: inner | B: G*N | C: G*N | dt: heads],
+    inner = heads * vdim."""
+
+    def __init__(self, width: int, heads: int, vdim: int, state: int,
+                 groups: int, norm_groups: int, taps: int, norm_eps: float,
+                 dtype):
+        super().__init__()
+        if heads % groups or (heads * vdim) % norm_groups:
+            raise ValueError("heads % groups and inner % norm_groups must be 0")
+        self.heads, self.vdim, self.state, self.groups = heads, vdim, state, \
+            groups
+        self.norm_groups, self.taps, self.eps = norm_groups, taps, norm_eps
+        self.inner = heads * vdim
+        self.conv_ch = self.inner + 2 * groups * state
+        self.in_width = 2 * self.inner + 2 * groups * state + heads
+        f32 = dict(dtype=torch.float32)
+        self.conv_w = nn.Parameter(torch.empty(self.conv_ch, taps, dtype=dtype))
+        self.conv_b = nn.Parameter(torch.zeros(self.conv_ch, dtype=dtype))
+        self.dt_bias = nn.Parameter(torch.zeros(heads, **f32))
+        self.A_log = nn.Parameter(torch.zeros(heads, **f32))
+        self.D = nn.Parameter(torch.ones(heads, **f32))
+        self.out_norm = nn.Parameter(torch.ones(self.inner, **f32))
+        self.o_proj = nn.Parameter(torch.empty(width, self.inner, dtype=dtype))
+
+    def cache_spec(self):
+        return CacheGroup((ConvState(self.conv_ch, self.taps),
+                           RecurrentState(self.heads, self.state, self.vdim)))
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        conv_state, ssm_state = cache
+        T, inner, gn = proj.shape[0], self.inner, self.groups * self.state
+        z = proj[:, :inner]
+        xbc_in = proj[:, inner:inner + self.conv_ch]
+        dt = proj[:, inner + self.conv_ch:self.in_width]
+        o = torch.empty(T, self.heads, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        for rows, cu_q, ctx, slots, _, _, max_len in _halves(meta, aux):
+            u = xbc_in[rows]
+            xbc = hops.short_conv(u, self.conv_w, self.conv_b, conv_state, 0,
+                                  slots, cu_q, ctx, 1, self.conv_ch,
+                                  act_silu=True)
+            hops.short_conv_state_(conv_state, u, slots, cu_q)
+            hops.gated_recurrence(
+                0, xbc[:, inner + gn:], xbc[:, inner:inner + gn],
+                xbc[:, :inner], dt[rows], self.dt_bias, self.A_log, self.D,
+                0.0, 1.0, ssm_state, slots, cu_q, ctx, self.groups, o[rows],
+                max_q_len=max_len)
+        y = hops.gated_group_norm(o.view(T, inner), self.out_norm, z, self.eps,
+                                  self.norm_groups, act_silu=True,
+                                  gate_first=True, out_dtype=proj.dtype)
+        return F.linear(y, self.o_proj)
+
+
+class CappedAttention(nn.Module):
+    """in_proj rows: [q: heads*dim | k: kv_heads*dim | v: kv_heads*vdim |
+    g: heads*vdim]."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int,
+                 vdim: int, taps: int, rot: Optional[dict], scale: float,
+                 softcap: Optional[float], dtype):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, \
+            dim, vdim
+        self.taps, self.scale = taps, float(scale)
+        self.softcap = float(softcap) if softcap else 0.0
+        self.rot_dims = int(rot["dims"]) if rot else 0
+        if self.rot_dims > dim or self.rot_dims % 2:
+            raise ValueError("rotary dims must be even and <= dim")
+        if self.rot_dims:
+            inv_freq, _ = scaled_rope_frequencies(
+                dict(base=rot["base"], dims=rot["dims"]))
+            self.register_buffer("inv_freq", inv_freq, persistent=False)
+        else:
+            self.inv_freq = None
+        self.cq, self.ck, self.cv = heads * dim, kv_heads * dim, \
+            kv_heads * vdim
+        self.conv_ch = self.cq + self.ck + self.cv
+        self.g_width = heads * vdim
+        self.in_width = self.conv_ch + self.g_width
+        # filters of q, k, v stacked in the order of the projection rows
+        self.conv_w = nn.Parameter(torch.empty(self.conv_ch, taps, dtype=dtype))
+        self.o_proj = nn.Parameter(torch.empty(width, self.g_width,
+                                               dtype=dtype))
+
+    def cache_spec(self):
+        return CacheGroup((ConvState(self.conv_ch, self.taps),
+                           PagedKV(self.kv_heads, self.dim, self.vdim)))
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        conv_state, (k_cache, v_cache) = cache
+        T, cq, ck = proj.shape[0], self.cq, self.ck
+        H, G = self.heads, self.kv_heads
+        qkv = proj[:, :self.conv_ch]
+        gate = proj[:, self.conv_ch:self.in_width]
+        o = torch.empty(T, H, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        rot = dict(rot_dims=self.rot_dims, inv_freq=self.inv_freq)
+        for rows, cu_q, ctx, slots, seq_lens, tables, _ in _halves(meta, aux):
+            u, pos = qkv[rows], positions[rows]
+            sm = meta.slot_mapping[rows]
+            q = hops.short_conv(u[:, :cq], self.conv_w[:cq], None, conv_state,
+                                0, slots, cu_q, ctx, H, self.dim,
+                                positions=pos, **rot)
+            hops.short_conv(u[:, cq:cq + ck], self.conv_w[cq:cq + ck], None,
+                            conv_state, cq, slots, cu_q, ctx, G, self.dim,
+                            positions=pos, cache=k_cache, slot_mapping=sm,
+                            **rot)
+            hops.short_conv(u[:, cq + ck:], self.conv_w[cq + ck:], None,
+                            conv_state, cq + ck, slots, cu_q, ctx, G,
+                            self.vdim, cache=v_cache, slot_mapping=sm)
+            hops.short_conv_state_(conv_state, u, slots, cu_q)
+            hops.capped_attn(q, k_cache, v_cache, tables, cu_q, seq_lens, H,
+                             self.scale, self.softcap, o[rows])
+        y = hops.norm_sigmoid_gate(o.view(T, self.g_width), None, gate, 0.0,
+                                   proj.dtype)
+        return F.linear(y, self.o_proj)
+
+
+class GatedLinearAttention(nn.Module):
+    """in_proj rows: [q: heads*dim | k: heads*dim | v: heads*vdim |
+    g: heads*vdim | a1: rank]; the decay logits are a2 (a1 h) + a2_b."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int,
+                 tau: float, rank: int, norm_eps: float, dtype):
+        super().__init__()
+        self.heads, self.dim, self.vdim = heads, dim, vdim
+        self.tau, self.rank, self.eps = float(tau), rank, norm_eps
+        self.qk_width, self.v_width = heads * dim, heads * vdim
+        self.in_width = 2 * self.qk_width + 2 * self.v_width + rank
+        self.a2 = nn.Parameter(torch.empty(self.qk_width, rank, dtype=dtype))
+        self.a2_b = nn.Parameter(torch.zeros(self.qk_width,
+                                             dtype=torch.float32))
+        self.out_norm = nn.Parameter(torch.ones(vdim, dtype=torch.float32))
+        self.o_proj = nn.Parameter(torch.empty(width, self.v_width,
+                                               dtype=dtype))
+
+    def cache_spec(self):
+        return RecurrentState(self.heads, self.dim, self.vdim)
+
+    def forward(self, proj, positions, state, meta: AttnMetadata, aux):
+        T, a, b = proj.shape[0], self.qk_width, self.v_width
+        q, k = proj[:, :a], proj[:, a:2 * a]
+        v = proj[:, 2 * a:2 * a + b]
+        gate = proj[:, 2 * a + b:2 * a + 2 * b]
+        z = F.linear(proj[:, 2 * a + 2 * b:self.in_width], self.a2)
+        o = torch.empty(T, self.heads, self.vdim, dtype=torch.float32,
+                        device=proj.device)
+        for rows, cu_q, ctx, slots, _, _, max_len in _halves(meta, aux):
+            hops.gated_recurrence(
+                1, q[rows], k[rows], v[rows], z[rows], self.a2_b, None, None,
+                1.0 / self.tau, self.dim ** -0.5, state, slots, cu_q, ctx,
+                self.heads, o[rows], max_q_len=max_len)
+        y = hops.gated_group_norm(o.view(T, b), self.out_norm, gate, self.eps,
+                                  self.heads, act_silu=True, gate_first=False,
+                                  out_dtype=proj.dtype)
+        return F.linear(y, self.o_proj)
+
+
+class ParallelMixer(nn.Module):
+    """Two mixers on the same input; the caller adds their outputs with the
+    weights `scales` (kept apart so the sum is taken in fp32)."""
+
+    def __init__(self, left: nn.Module, right: nn.Module, left_scale: float,
+                 right_scale: float):
+        super().__init__()
+        self.left, self.right = left, right
+        self.scales = (float(left_scale), float(right_scale))
+        self.in_width = left.in_width + right.in_width
+
+    def cache_spec(self):
+        return CacheGroup((self.left.cache_spec(), self.right.cache_spec()))
+
+    def forward(self, proj, positions, cache, meta: AttnMetadata, aux):
+        lw = self.left.in_width
+        return (self.left(proj[:, :lw], positions, cache[0], meta, aux),
+                self.right(proj[:, lw:self.in_width], positions, cache[1],
+                           meta, aux))

@@ -21,11 +21,14 @@ def create_model(cfg: ModelConfig, dtype=torch.bfloat16):
     if cfg.architecture == "pugovik":
         from .pugovik import PugovikForCausalLM
         return PugovikForCausalLM(cfg, dtype=dtype)
+    if cfg.architecture == "dunusun":
+        from .dunusun import DunusunForCausalLM
+        return DunusunForCausalLM(cfg, dtype=dtype)
     raise ValueError(f"unknown architecture {cfg.architecture}")
 
 
 def required_extensions(cfg: ModelConfig):
     """In-tree HIP extension modules the model's GPU path loads."""
-    if cfg.architecture == "pugovik":
+    if cfg.architecture in ("pugovik", "dunusun"):
         return ["_ops_hybrid"]
     return ["_ops"]

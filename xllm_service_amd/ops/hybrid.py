@@ -148,3 +148,113 @@ def moe_combine(y, rows, wts, tokens: int):
         return out
     yy = y.reshape(-1, width).float()[rows.long()]          # [T, top, W]
     return (yy * wts[:, :, None]).sum(1)
+
+
+# ---- residual streams, short convolutions, gated recurrences ---------------
+def streams_mix_norm(x, w_in: Optional[torch.Tensor], g, b, eps: float,
+                     out_dtype):
+    """Layer norm (weight g, bias b) of sum_s w_in[s] x[:, s]; x fp32
+    [T, S, W] -> [T, W]."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], x.shape[2], dtype=out_dtype,
+                          device=x.device)
+        _hyb().streams_mix_norm(out, x, w_in, g, b, eps)
+        return out
+    return ref.streams_mix_norm(x, w_in, g, b, eps, out_dtype)
+
+
+def streams_update_(x, mix, w_out, y1, a1: float = 1.0, y2=None,
+                    a2: float = 0.0):
+    """x[:, j] <- sum_s mix[s, j] x[:, s] + w_out[j] (a1 y1 + a2 y2), in
+    place on the fp32 streams [T, S, W]; mix / w_out None = identity / 1."""
+    if x.is_cuda:
+        _hyb().streams_update(x, mix, w_out, y1, a1, y2, a2)
+        return x
+    return ref.streams_update(x, mix, w_out, y1, a1, y2, a2)
+
+
+def relu_sq_(x):
+    if x.is_cuda:
+        _hyb().relu_sq(x)
+        return x
+    return x.copy_(torch.relu(x.float()).pow(2).to(x.dtype))
+
+
+def softcap(x, cap: float):
+    """fp32 cap * tanh(x / cap)."""
+    if x.is_cuda:
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        _hyb().softcap(out, x.contiguous(), cap)
+        return out
+    return cap * torch.tanh(x.float() / cap)
+
+
+def short_conv(x, w, bias, state, state_off: int, slots, cu_q, ctx_lens,
+               heads: int, hd: int, *, act_silu: bool = False,
+               rot_dims: int = 0, positions=None, inv_freq=None,
+               cache=None, slot_mapping=None):
+    """Short causal convolution with carried inputs (see ref.short_conv).
+    With `cache` [blocks, heads, block, hd] the result is scattered to the
+    tokens' slots and None is returned; else a new [T, heads*hd] tensor."""
+    if x.is_cuda:
+        out = None
+        if cache is None:
+            out = torch.empty(x.shape[0], heads * hd, dtype=x.dtype,
+                              device=x.device)
+        _hyb().short_conv(out, cache, slot_mapping, x, w, bias, state,
+                          state_off, slots, cu_q, ctx_lens, heads, hd,
+                          act_silu, rot_dims, positions, inv_freq)
+        return out
+    out = ref.short_conv(x, w, bias, state, state_off, slots, cu_q, ctx_lens,
+                         heads, hd, act_silu, rot_dims, positions, inv_freq)
+    if cache is None:
+        return out
+    ref.store_paged(out, cache, slot_mapping)
+    return None
+
+
+def short_conv_state_(state, x, slots, cu_q):
+    """After every reader of the old state ran: keep the last taps-1 rows."""
+    if state.shape[1] == 0:
+        return
+    if x.is_cuda:
+        _hyb().short_conv_state(state, x, slots, cu_q)
+        return
+    ref.short_conv_state(state, x, slots, cu_q)
+
+
+def gated_recurrence(kind: int, q, k, v, g, p0, p1, p2, c0: float, c1: float,
+                     state, slots, cu_q, ctx_lens, groups: int, out,
+                     max_q_len: int = 0):
+    """out fp32 [T, H, Dv] (written); see ref.gated_recurrence."""
+    if q.is_cuda:
+        _hyb().gated_recurrence(kind, out, q, k, v, g, p0, p1, p2, c0, c1,
+                                state, slots, cu_q, ctx_lens, groups,
+                                max_q_len)
+        return out
+    out.copy_(ref.gated_recurrence(kind, q, k, v, g, p0, p1, p2, c0, c1,
+                                   state, slots, cu_q, ctx_lens, groups))
+    return out
+
+
+def gated_group_norm(o, w, gate, eps: float, groups: int, *, act_silu: bool,
+                     gate_first: bool, out_dtype):
+    if o.is_cuda:
+        out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+        _hyb().gated_group_norm(out, o, w, gate, eps, groups, act_silu,
+                                gate_first)
+        return out
+    return ref.gated_group_norm(o, w, gate, eps, groups, act_silu,
+                                gate_first, out_dtype)
+
+
+def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens,
+                heads: int, scale: float, cap: float, out):
+    """out fp32 [T, heads, Dv] (written). cu_q None: decode rows."""
+    if q.is_cuda:
+        _hyb().capped_attn(out, q, k_cache, v_cache, block_tables, cu_q,
+                           seq_lens, heads, scale, cap)
+        return out
+    out.copy_(ref.capped_attn(q, k_cache, v_cache, block_tables, cu_q,
+                              seq_lens, heads, scale, cap))
+    return out

@@ -301,3 +301,181 @@ def moe_route(h, w_router, top, n_groups, keep):
 def silu_mul(x):
     """[..., 2F] -> silu(x[..., :F]) * x[..., F:], dtype preserved."""
     return silu_and_mul(x)
+
+
+# ---------------------------------------------------------------------------
+# Residual streams, short convolutions with state, data-dependent linear
+# recurrences, soft-capped paged attention. fp32 throughout.
+# ---------------------------------------------------------------------------
+def streams_mix_norm(x, w_in, g, b, eps, out_dtype):
+    """x fp32 [T, S, W] -> layer norm of sum_s w_in[s] x[:, s], times g
+    plus b, [T, W]. w_in None: plain sum."""
+    u = x.sum(1) if w_in is None else torch.einsum("tsw,s->tw", x, w_in)
+    mu = u.mean(-1, keepdim=True)
+    var = (u - mu).pow(2).mean(-1, keepdim=True)
+    return ((u - mu) * torch.rsqrt(var + eps) * g + b).to(out_dtype)
+
+
+def streams_update(x, mix, w_out, y1, a1, y2, a2):
+    """x[:, j] <- sum_s mix[s, j] x[:, s] + w_out[j] (a1 y1 + a2 y2)."""
+    S = x.shape[1]
+    y = a1 * y1.float()
+    if y2 is not None:
+        y = y + a2 * y2.float()
+    m = torch.eye(S) if mix is None else mix
+    wo = torch.ones(S) if w_out is None else w_out
+    x.copy_(torch.einsum("tsw,sj->tjw", x, m) + wo[None, :, None] * y[:, None])
+    return x
+
+
+def _seq_ranges(T, slots, cu_q):
+    n = len(slots)
+    if cu_q is None:
+        return [(s, s, s + 1) for s in range(n)]
+    return [(s, int(cu_q[s]), int(cu_q[s + 1])) for s in range(n)]
+
+
+def short_conv(x, w, bias, state, state_off, slots, cu_q, ctx_lens, heads, hd,
+               act_silu, rot_dims, positions, inv_freq):
+    """Causal per-channel convolution of x [T, C] (C = heads*hd) with w
+    [C, taps]; earlier inputs of a sequence come from state[slot, i,
+    state_off:state_off+C] (the input of position ctx - (taps-1) + i), zeros
+    before position 0. Optional bias, SiLU, and an interleaved rotary turn of
+    the first rot_dims channels of every head. Returns [T, C] in x's dtype."""
+    T, C = x.shape
+    taps = w.shape[1]
+    K1 = taps - 1
+    out = torch.zeros(T, C, dtype=torch.float32)
+    wf = w.float()
+    for s, t0, t1 in _seq_ranges(T, slots, cu_q):
+        ctx, slot = int(ctx_lens[s]), int(slots[s])
+        hist = torch.zeros(K1, C, dtype=torch.float32)
+        if slot >= 0 and K1:
+            hist = state[slot, :, state_off:state_off + C].float().clone()
+        for i in range(K1):                 # positions before the sequence
+            if ctx - K1 + i < 0:
+                hist[i] = 0.0
+        u = torch.cat([hist, x[t0:t1].float()], 0)
+        for j in range(taps):
+            out[t0:t1] += wf[:, j] * u[j:j + (t1 - t0)]
+    if bias is not None:
+        out += bias.float()
+    if act_silu:
+        out = torch.nn.functional.silu(out)
+    if rot_dims:
+        o3 = out.view(T, heads, hd).to(x.dtype)
+        out = rope_interleaved(o3, positions, inv_freq, 1.0, rot_dims) \
+            .reshape(T, C)
+    return out.to(x.dtype)
+
+
+def short_conv_state(state, x, slots, cu_q):
+    """Move every sequence's convolution state past this step's rows."""
+    K1 = state.shape[1]
+    if K1 == 0:
+        return
+    for s, t0, t1 in _seq_ranges(x.shape[0], slots, cu_q):
+        slot = int(slots[s])
+        if slot < 0:
+            continue
+        u = torch.cat([state[slot], x[t0:t1].to(state.dtype)], 0)
+        state[slot] = u[-K1:]
+
+
+def gated_recurrence(kind, q, k, v, g, p0, p1, p2, c0, c1, state, slots, cu_q,
+                     ctx_lens, groups):
+    """S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t (+ skip v_t);
+    kind 0 (selective state space): dt = softplus(g + p0), a = exp(-exp(p1)
+    dt) per head, k = dt * k, skip = p2; q/k shared by the heads of a group.
+    kind 1 (gated linear attention): a = sigmoid(g + p0)^c0 per key channel,
+    q scaled by c1. state fp32 [slots, H, D, Dv]; returns fp32 [T, H, Dv]."""
+    H, D, Dv = state.shape[1:]
+    T = q.shape[0]
+    per = H // groups
+    qf = q.float().view(T, groups, D).repeat_interleave(per, 1)
+    kf = k.float().view(T, groups, D).repeat_interleave(per, 1)
+    vf = v.float().view(T, H, Dv)
+    if kind == 0:
+        dt = torch.nn.functional.softplus(g.float() + p0, threshold=30.0)
+        a = torch.exp(-torch.exp(p1) * dt)[:, :, None].expand(T, H, D)
+        kf = kf * dt[:, :, None]
+    else:
+        z = g.float() + p0
+        a = torch.exp(-torch.nn.functional.softplus(-z, threshold=30.0) * c0) \
+            .view(T, H, D)
+        qf = qf * c1
+    out = torch.zeros(T, H, Dv, dtype=torch.float32)
+    for s, t0, t1 in _seq_ranges(T, slots, cu_q):
+        slot = int(slots[s])
+        if slot >= 0 and int(ctx_lens[s]) > 0:
+            S = state[slot].clone()
+        else:
+            S = torch.zeros(H, D, Dv, dtype=torch.float32)
+        for t in range(t0, t1):
+            S = a[t][:, :, None] * S + kf[t][:, :, None] * vf[t][:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        if slot >= 0:
+            state[slot] = S
+    if kind == 0 and p2 is not None:
+        out = out + p2[None, :, None] * vf
+    return out
+
+
+def gated_group_norm(o, w, gate, eps, groups, act_silu, gate_first,
+                     out_dtype):
+    """RMS norm over `groups` equal parts of fp32 o [rows, n], times w (n
+    or n/groups entries, repeating), with gate silu/sigmoid applied before
+    or after the norm."""
+    act = torch.nn.functional.silu if act_silu else torch.sigmoid
+    a = act(gate.float())
+    z = o.float() * a if gate_first else o.float()
+    rows, n = z.shape
+    zg = z.view(rows, groups, n // groups)
+    zg = zg * torch.rsqrt(zg.pow(2).mean(-1, keepdim=True) + eps)
+    wf = w.float()
+    if wf.numel() != n:
+        wf = wf.repeat(groups)
+    z = zg.reshape(rows, n) * wf
+    if not gate_first:
+        z = z * a
+    return z.to(out_dtype)
+
+
+def store_paged(x, cache, slot_mapping):
+    """x [T, heads*hd] into cache [blocks, heads, block, hd] at the slots."""
+    nb, heads, bs, hd = cache.shape
+    ok = slot_mapping >= 0
+    sl = slot_mapping[ok]
+    cache[sl // bs, :, sl % bs] = x[ok].view(-1, heads, hd).to(cache.dtype)
+
+
+def capped_attn(q, k_cache, v_cache, block_tables, cu_q, seq_lens, heads,
+                scale, cap):
+    """Causal softmax attention of q [T, heads*D] over the paged caches
+    [blocks, n_kv, block, D|Dv]; scores scale * q.k, then cap * tanh(. /
+    cap) when cap > 0. Returns fp32 [T, heads, Dv]."""
+    T = q.shape[0]
+    nb, n_kv, bs, D = k_cache.shape
+    Dv = v_cache.shape[3]
+    per = heads // n_kv
+    out = torch.zeros(T, heads, Dv, dtype=torch.float32)
+    if cu_q is None:
+        cu_q = torch.arange(T + 1, dtype=torch.int32)
+    for s in range(len(seq_lens)):
+        q0, q1 = int(cu_q[s]), int(cu_q[s + 1])
+        L = int(seq_lens[s])
+        ctx = L - (q1 - q0)
+        nblk = (L + bs - 1) // bs
+        idx = block_tables[s][:nblk].long()
+        kk = k_cache[idx].float().permute(1, 0, 2, 3).reshape(n_kv, -1, D)[:, :L]
+        vv = v_cache[idx].float().permute(1, 0, 2, 3).reshape(n_kv, -1, Dv)[:, :L]
+        kk = kk.repeat_interleave(per, 0)
+        vv = vv.repeat_interleave(per, 0)
+        qq = q[q0:q1].float().view(q1 - q0, heads, D)
+        sc = torch.einsum("thd,hld->thl", qq, kk) * scale
+        if cap and cap > 0:
+            sc = cap * torch.tanh(sc / cap)
+        mask = torch.arange(L)[None, :] > (ctx + torch.arange(q1 - q0))[:, None]
+        sc = sc.masked_fill(mask[:, None, :], float("-inf"))
+        out[q0:q1] = torch.einsum("thl,hlv->thv", torch.softmax(sc, -1), vv)
+    return out
