@@ -56,7 +56,8 @@ ext_modules = [
             for f in ("bindings.cpp", "norms.hip", "latent_attn.hip",
                       "latent_attn_mfma.hip", "decay_attn.hip", "moe.hip",
                       "streams.hip", "short_conv.hip",
-                      "gated_recurrence.hip", "capped_attn.hip")
+                      "gated_recurrence.hip", "capped_attn.hip",
+                      "capped_attn_mfma.hip")
         ],
         extra_compile_args={
             "cxx": ["-O3", "-std=c++17"],

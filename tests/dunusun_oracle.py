@@ -25,7 +25,6 @@ import math
 import os
 import struct
 
-import numpy as np
 import torch
 
 F64 = torch.float64
@@ -307,7 +306,8 @@ def make_weights(cfg, seed=0, gain=1.0):
         if lc.get("mlp") is not None:
             out[p + "mlp.up"] = rnd(lc["mlp"]["ff"], W)
             out[p + "mlp.down"] = rnd(W, lc["mlp"]["ff"])
-    return out
+    # what the file holds is what the oracle sees
+    return {k: v.bfloat16().float() for k, v in out.items()}
 
 
 def file_config(cfg):

@@ -7,6 +7,7 @@
 #include <ATen/hip/HIPContext.h>
 
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 
 namespace xllm {
@@ -76,6 +77,12 @@ void launch_gated_recurrence(int, float*, const T*, const T*, const T*,
 template <typename T>
 void launch_gated_group_norm(T*, const float*, const float*, int, const T*,
                              long, float, int, int, int, int, int,
+                             hipStream_t);
+int capped_attn_mfma_class(int D, int Dv);
+void launch_capped_attn_mfma(float*, float*, float*, const unsigned short*,
+                             const unsigned short*, const unsigned short*,
+                             const int*, const int*, const int*, int, int, int,
+                             int, int, int, int, int, float, float, long, int,
                              hipStream_t);
 template <typename T>
 void launch_capped_attn(float*, const T*, const T*, const T*, const int*,
@@ -644,6 +651,35 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     cu = ptr<int>(*cu_q);
   } else {
     TORCH_CHECK(n_seqs == T, "decode: one sequence per token");
+  }
+  // bf16: MFMA kernel when the sizes fit one of its instantiations
+  if (is_bf16(q) && hy::capped_attn_mfma_class(D, Dv) != 0 &&
+      q.stride(0) % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
+    int n_part = 1;
+    Tensor ws_acc, ws_ml;
+    if (cu == nullptr) {
+      // decode: split the context over workgroups when (token, key/value
+      // head) pairs alone do not fill the chip; sizes known on the host only
+      const int per = heads / n_kv;
+      const int rows_wg = per <= 16 ? 16 : per <= 32 ? 32 : 64;
+      const long wgs = (long)T * n_kv * ((per + rows_wg - 1) / rows_wg);
+      const long max_tiles = ((long)block_tables.size(1) * bs + 31) / 32;
+      n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
+                                   std::max<long>(1, 256 / wgs));
+      n_part = std::max(n_part, 1);
+    }
+    if (n_part > 1) {
+      ws_acc = torch::empty({(long)T * heads * n_part, (long)Dv}, out.options());
+      ws_ml = torch::empty({(long)T * heads * n_part, 2}, out.options());
+    }
+    hy::launch_capped_attn_mfma(
+        ptr<float>(out), n_part > 1 ? ptr<float>(ws_acc) : nullptr,
+        n_part > 1 ? ptr<float>(ws_ml) : nullptr, ptr<bf>(q), ptr<bf>(k_cache),
+        ptr<bf>(v_cache), ptr<int>(block_tables), cu, ptr<int>(seq_lens), T,
+        n_seqs, heads, n_kv, D, Dv, bs, block_tables.size(1), scale, cap,
+        q.stride(0), n_part, cur());
+    return;
   }
   TORCH_CHECK((size_t)4 * D * 4 <= 64 * 1024, "query row too wide for LDS");
   if (is_f32(q))
