@@ -66,6 +66,10 @@ def parse_args():
                          "llama stacks (one GPU; prints one JSON line per "
                          "measurement, not the headline record)")
     ap.add_argument("--hybrid-sizes", default="2k,4k")
+    ap.add_argument("--hybrid-family", default="pugovik",
+                    choices=("pugovik", "dunusun"),
+                    help="which hybrid stack --mode hybrid measures beside "
+                         "the equal-size llama stack")
     ap.add_argument("--model", default="llama-3-8b")
     ap.add_argument("--concurrency", type=int, default=128,
                     help="ramp/calibration concurrency per decode GPU "
@@ -239,17 +243,151 @@ def _hybrid_kernels(size, device, T, batch, ctx):
     return out
 
 
+def _dunusun_kernels(size, device, T, batch, ctx):
+    """Achieved rates of the Dunusun mixer kernels at one layer's shapes,
+    beside the like kernels of the pugovik / llama stacks of that size."""
+    from xllm_service_amd import ops
+    from xllm_service_amd.models.config import get_config
+    from xllm_service_amd.ops import hybrid as hops
+    dc, pc, lc = (get_config(f"{f}-{size}") for f in ("dunusun", "pugovik",
+                                                       "llama"))
+    par = next(l.mixer for l in dc.layers if l.type == "parallel")
+    ssm = next(l.mixer for l in dc.layers if l.type == "mamba2")
+    lin = next(l.mixer for l in pc.layers if l.type == "lightning")
+    bf = dict(dtype=torch.bfloat16, device=device)
+    f32 = dict(dtype=torch.float32, device=device)
+    i32 = dict(dtype=torch.int32, device=device)
+    out = []
+    nblk = (max(T, ctx) + 15) // 16
+    tab = torch.arange(batch * nblk, **i32).view(batch, nblk)
+    cu = torch.tensor([0, T], **i32)
+    sl = torch.tensor([T], **i32)
+    sld = torch.full((batch,), ctx, **i32)
+    z1 = torch.zeros(1, **i32)
+    sls = torch.arange(batch, **i32)
+    cx = torch.full((batch,), ctx, **i32)
+    # ---- soft-capped attention vs paged attention ------------------------
+    L = par["left"]
+    H, G, D, Dv = L["heads"], L["kv_heads"], L["dim"], L["vdim"]
+    kc = torch.randn(batch * nblk, G, 16, D, **bf)
+    vc = torch.randn(batch * nblk, G, 16, Dv, **bf)
+    q = torch.randn(T, H * D, **bf)
+    o = torch.empty(T, H, Dv, **f32)
+    t = _time_gpu(lambda: hops.capped_attn(q, kc, vc, tab[:1], cu, sl, H,
+                                           L["scale"], L["softcap"], o), 3, 1)
+    out.append(("capped_attn prefill", t,
+                2.0 * H * (D + Dv) * T * (T + 1) / 2 / t / 1e12, "TFLOP/s"))
+    qd = torch.randn(batch, H * D, **bf)
+    od = torch.empty(batch, H, Dv, **f32)
+    t = _time_gpu(lambda: hops.capped_attn(qd, kc, vc, tab, None, sld, H,
+                                           L["scale"], L["softcap"], od))
+    out.append(("capped_attn decode", t,
+                batch * ctx * G * (D + Dv) * 2 / t / 1e9, "GB/s"))
+    Hq, Hk, Dl = lc.num_heads, lc.num_kv_heads, lc.head_dim
+    kl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    vl = torch.randn(batch * nblk, Hk, 16, Dl, **bf)
+    ql = torch.randn(T, Hq, Dl, **bf)
+    if Dl == 128:
+        t = _time_gpu(lambda: ops.paged_attn_prefill(ql, kl, vl, tab[:1], cu,
+                                                     sl, 0.1), 3, 1)
+        out.append(("paged_attn prefill (llama)", t,
+                    4.0 * Hq * Dl * T * (T + 1) / 2 / t / 1e12, "TFLOP/s"))
+    qld = torch.randn(batch, Hq, Dl, **bf)
+    t = _time_gpu(lambda: ops.paged_attn_decode(qld, kl, vl, tab, sld, 0.1))
+    out.append(("paged_attn decode (llama)", t,
+                batch * ctx * Hk * Dl * 2 * 2 / t / 1e9, "GB/s"))
+    # ---- gated recurrences vs decayed linear attention -------------------
+    def recur(kind, Hh, Gg, Dk, Dvv, tokens, slots, cuq, ctxl):
+        qq = torch.randn(tokens, Gg * Dk, **bf)
+        kk = torch.randn(tokens, Gg * Dk, **bf)
+        vv = torch.randn(tokens, Hh * Dvv, **bf)
+        gg = torch.randn(tokens, Hh if kind == 0 else Hh * Dk, **bf)
+        st = torch.zeros(batch, Hh, Dk, Dvv, **f32)
+        p0 = torch.zeros(Hh if kind == 0 else Hh * Dk, **f32)
+        p1 = torch.zeros(Hh, **f32) if kind == 0 else None
+        oo = torch.empty(tokens, Hh, Dvv, **f32)
+        return lambda: hops.gated_recurrence(
+            kind, qq, kk, vv, gg, p0, p1, p1, 0.06, 0.1, st, slots, cuq, ctxl,
+            Gg, oo, max_q_len=tokens)
+    Hs, P, N, Gs = ssm["heads"], ssm["vdim"], ssm["state"], ssm["groups"]
+    R = par["right"]
+    for label, kind, Hh, Gg, Dk, Dvv in (
+            ("ssm", 0, Hs, Gs, N, P),
+            ("gla", 1, R["heads"], R["heads"], R["dim"], R["vdim"])):
+        t = _time_gpu(recur(kind, Hh, Gg, Dk, Dvv, T, z1, cu, z1), 3, 1)
+        out.append((f"gated_recurrence {label} prefill", t,
+                    4.0 * Hh * Dk * Dvv * T / t / 1e12,
+                    "TFLOP/s (recurrence form)"))
+        t = _time_gpu(recur(kind, Hh, Gg, Dk, Dvv, batch, sls, None, cx))
+        out.append((f"gated_recurrence {label} decode", t,
+                    batch * Hh * Dk * Dvv * 4 * 2 / t / 1e9, "GB/s"))
+    Hh, Dk, Dvv = lin["heads"], lin["dim"], lin["vdim"]
+    dec = torch.tensor(lin["decay"], **f32)
+    st = torch.zeros(batch, Hh, Dk, Dvv, **f32)
+    qkv = torch.randn(T, 2 * Hh * Dk + Hh * Dvv, **bf)
+    oo = torch.empty(T, Hh, Dvv, **f32)
+    t = _time_gpu(lambda: hops.decay_attn(
+        qkv[:, :Hh * Dk], qkv[:, Hh * Dk:2 * Hh * Dk], qkv[:, 2 * Hh * Dk:],
+        dec, st, z1, cu, z1, oo), 3, 1)
+    out.append(("decay_attn prefill (pugovik)", t,
+                4.0 * Hh * Dk * Dvv * T / t / 1e12,
+                "TFLOP/s (recurrence form)"))
+    qkvd = torch.randn(batch, 2 * Hh * Dk + Hh * Dvv, **bf)
+    ood = torch.empty(batch, Hh, Dvv, **f32)
+    t = _time_gpu(lambda: hops.decay_attn(
+        qkvd[:, :Hh * Dk], qkvd[:, Hh * Dk:2 * Hh * Dk], qkvd[:, 2 * Hh * Dk:],
+        dec, st, sls, None, cx, ood))
+    out.append(("decay_attn decode (pugovik)", t,
+                batch * Hh * Dk * Dvv * 4 * 2 / t / 1e9, "GB/s"))
+    # ---- short convolution -------------------------------------------------
+    C, taps = Hs * P + 2 * Gs * N, ssm["conv"]
+    xin = torch.randn(T, C, **bf)
+    cw, cb = torch.randn(C, taps, **bf), torch.randn(C, **bf)
+    cst = torch.zeros(batch, taps - 1, C, **bf)
+    t = _time_gpu(lambda: hops.short_conv(xin, cw, cb, cst, 0, z1, cu, z1, 1,
+                                          C, act_silu=True))
+    out.append(("short_conv+silu", t, T * C * 4 / t / 1e9, "GB/s"))
+    # ---- streams and norms -------------------------------------------------
+    Wd, S = dc.hidden_size, dc.streams or 1
+    xs = torch.randn(T, S, Wd, **f32)
+    w = torch.ones(Wd, **f32)
+    wi = torch.ones(S, **f32)
+    mix = torch.eye(S, **f32)
+    t = _time_gpu(lambda: hops.streams_mix_norm(xs, wi, w, w, 1e-6,
+                                                torch.bfloat16))
+    out.append(("streams_mix_norm", t, T * Wd * (4 * S + 2) / t / 1e9,
+                "GB/s"))
+    y = torch.randn(T, Wd, **bf)
+    t = _time_gpu(lambda: hops.streams_update_(xs, mix, wi, y, 1.0, y, 1.0))
+    out.append(("streams_update", t, T * Wd * (8 * S + 4) / t / 1e9, "GB/s"))
+    x1 = torch.randn(T, Wd, **f32)
+    t = _time_gpu(lambda: hops.group_rmsnorm(x1, w, 1e-6, pc.norm_groups,
+                                             torch.bfloat16))
+    out.append(("group_rmsnorm fp32->bf16 (pugovik)", t,
+                T * Wd * 6 / t / 1e9, "GB/s"))
+    gt = torch.randn(T, Wd, **bf)
+    t = _time_gpu(lambda: hops.gated_norm_residual(x1, y, gt, w, w, w, 0.5,
+                                                   1e-6, pc.norm_groups))
+    out.append(("gated_norm_residual (pugovik)", t, T * Wd * 12 / t / 1e9,
+                "GB/s"))
+    return out
+
+
 def run_hybrid_mode(args, device):
     assert torch.cuda.is_available(), "hybrid mode measures the HIP path"
+    kernels = _hybrid_kernels
+    fams = ("pugovik", "llama")
+    if args.hybrid_family == "dunusun":
+        kernels = _dunusun_kernels
+        fams = ("dunusun", "pugovik", "llama")
     for size in args.hybrid_sizes.split(","):
         T, batch, ctx = 4096, 32, 2048
-        for name, t, rate, unit in _hybrid_kernels(size, device, T, batch,
-                                                   ctx):
+        for name, t, rate, unit in kernels(size, device, T, batch, ctx):
             print(json.dumps(dict(kind="kernel", size=size, kernel=name,
                                   ms=round(t * 1e3, 4), rate=round(rate, 2),
                                   unit=unit, tokens=T, batch=batch, ctx=ctx)),
                   flush=True)
-        for fam in ("pugovik", "llama"):
+        for fam in fams:
             pre, dec = _hybrid_end_to_end(f"{fam}-{size}", device, T, batch,
                                           1024, args.steps)
             print(json.dumps(dict(kind="end_to_end", model=f"{fam}-{size}",

@@ -139,7 +139,8 @@ def test_residual_after_every_layer_run(root, target, name):
     toks = _tokens(cfg, 21, 5)
     seen = []
     hooks = [l.register_forward_hook(lambda m, i, o: seen.append(
-        o.detach().float().sum(1).cpu().clone())) for l in eng.model.layers]
+        o[0].detach().float().sum(1).cpu().clone()))
+        for l in eng.model.layers]
     eng.score_step([("a", toks, [0])], finished=["a"])
     for h in hooks:
         h.remove()

@@ -65,6 +65,15 @@ def test_streams_read_and_write(target, S, W):
         sum(mix[s, j].to(F64) * x[:, s].to(F64) for s in range(S))
         + w_out[j].to(F64) * y for j in range(S)], 1)
     _close(xd, want, ("", torch.float32), "write")
+    # the write fused with the next sublayer's read
+    xf = x.clone().to(dev)
+    w2 = torch.randn(S, generator=g)
+    h = hops.streams_update_mix_norm_(xf, mix.to(dev), w_out.to(dev),
+                                      y1.to(dev), 0.7, y2.to(dev), -1.3,
+                                      w2.to(dev), nw.to(dev), nb.to(dev), 1e-5)
+    _close(xf, want, ("", torch.float32), "fused write")
+    u = torch.einsum("tsw,s->tw", want, w2.to(F64))
+    _close(h, o_layernorm(u, nw.to(F64), nb.to(F64), 1e-5), target, "fused")
     # identity mixing = the plain residual sum
     x1 = x[:, :1].clone().to(dev)
     hops.streams_update_(x1, None, None, y1.to(dev))
@@ -327,6 +336,22 @@ def test_recurrence_long_chunks(target, kind, fast):
     _recurrence_case(target, kind, H, G, 18, 16, [700, 5],
                      [[(0, 300), (1, 4)], [(0, 1), (1, 1)], [(0, 399)]],
                      seed=20 + kind, fast_decay=fast)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("kind", [0, 1])
+@pytest.mark.parametrize("cols", ["1", "4"])
+def test_recurrence_wide_values(target, kind, cols, monkeypatch):
+    """Wide value rows, with one and with four columns per thread (the
+    kernel picks by grid size; the knob fixes it), whole chunks and pieces;
+    a value width that leaves the last column group part empty."""
+    monkeypatch.setenv("XLLM_RECURRENCE_COLS", cols)
+    H, G = (2, 1) if kind == 0 else (2, 2)
+    _recurrence_case(target, kind, H, G, 12, 72, [330, 40],
+                     [[(0, 290), (1, 39)], [(0, 1), (1, 1)], [(0, 39)]],
+                     seed=30 + kind)
+    _recurrence_case(target, kind, H, G, 33, 50, [21],
+                     [[(0, 20)], [(0, 1)]], seed=40 + kind)
 
 
 # ------------------------------------------------------- soft-capped attention

@@ -57,6 +57,11 @@ template <typename T>
 void launch_streams_update(float*, const float*, const float*, const T*, float,
                            const T*, float, long, int, int, hipStream_t);
 template <typename T>
+void launch_streams_update_mix_norm(T*, float*, const float*, const float*,
+                                    const T*, float, const T*, float,
+                                    const float*, const float*, const float*,
+                                    float, int, int, int, hipStream_t);
+template <typename T>
 void launch_relu_sq(T*, long, hipStream_t);
 template <typename T>
 void launch_softcap(float*, const T*, float, long, hipStream_t);
@@ -425,6 +430,42 @@ void streams_update(Tensor x, c10::optional<Tensor> mix,
     hy::launch_streams_update<bf>(ptr<float>(x), mp, op, ptr<bf>(y1), a1, (const bf*)y2p, a2, T, S, W, cur());
 }
 
+// streams_update followed by streams_mix_norm of the new values, one pass
+void streams_update_mix_norm(Tensor out, Tensor x, c10::optional<Tensor> mix,
+                             c10::optional<Tensor> w_out, Tensor y1, double a1,
+                             c10::optional<Tensor> y2, double a2,
+                             c10::optional<Tensor> w_in, Tensor g, Tensor b,
+                             double eps) {
+  CHK_ACT(out); CHK_F32C(x); CHK_ACT(y1); CHK_F32C(g); CHK_F32C(b);
+  TORCH_CHECK(x.dim() == 3 && y1.is_contiguous() && out.is_contiguous() &&
+              out.dim() == 2 && out.dtype() == y1.dtype());
+  const int T = x.size(0), S = x.size(1), W = x.size(2);
+  TORCH_CHECK(S >= 1 && S <= 8 && y1.numel() == (long)T * W &&
+              out.size(0) == T && out.size(1) == W && g.numel() == W &&
+              b.numel() == W);
+  TORCH_CHECK((size_t)W * 4 <= 60 * 1024, "width too large for LDS");
+  auto opt = [&](const c10::optional<Tensor>& t, long n) -> const float* {
+    if (!t.has_value()) return nullptr;
+    CHK_F32C(*t);
+    TORCH_CHECK(t->numel() == n);
+    return ptr<float>(*t);
+  };
+  const float* mp = opt(mix, (long)S * S);
+  const float* op = opt(w_out, S);
+  const float* ip = opt(w_in, S);
+  const void* y2p = nullptr;
+  if (y2.has_value()) {
+    CHK_ACT(*y2);
+    TORCH_CHECK(y2->is_contiguous() && y2->numel() == (long)T * W &&
+                y2->dtype() == y1.dtype());
+    y2p = y2->data_ptr();
+  }
+  if (is_f32(y1))
+    hy::launch_streams_update_mix_norm<float>(ptr<float>(out), ptr<float>(x), mp, op, ptr<float>(y1), a1, (const float*)y2p, a2, ip, ptr<float>(g), ptr<float>(b), eps, T, S, W, cur());
+  else
+    hy::launch_streams_update_mix_norm<bf>(ptr<bf>(out), ptr<float>(x), mp, op, ptr<bf>(y1), a1, (const bf*)y2p, a2, ip, ptr<float>(g), ptr<float>(b), eps, T, S, W, cur());
+}
+
 void relu_sq(Tensor x) {
   CHK_ACT(x);
   TORCH_CHECK(x.is_contiguous());
@@ -590,6 +631,11 @@ void gated_recurrence(long kind, Tensor out, Tensor q, Tensor k, Tensor v,
   if (cu != nullptr) {
     const long bound = max_q_len > 0 ? std::min<long>(max_q_len, T) : T;
     const long per_seq = (long)H * D * Dv * 4;
+    // few heads: shorter pieces, so that the piece-parallel passes still
+    // fill the chip
+    while (chunk > 32 &&
+           (bound + chunk - 1) / chunk * n_seqs * H * ((Dv + 63) / 64) < 1024)
+      chunk /= 2;
     while ((bound + chunk - 1) / chunk * n_seqs * per_seq > (1L << 31))
       chunk *= 2;                             // keep the scratch under 2 GiB
     if (bound >= 2L * chunk) {
@@ -660,14 +706,19 @@ void capped_attn(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     Tensor ws_acc, ws_ml;
     if (cu == nullptr) {
       // decode: split the context over workgroups when (token, key/value
-      // head) pairs alone do not fill the chip; sizes known on the host only
+      // head) pairs alone do not fill the chip; sizes known on the host only.
+      // About four workgroups per CU measured best (batch 8..128, 1k-4k
+      // context, 4-8 key/value heads).
       const int per = heads / n_kv;
       const int rows_wg = per <= 16 ? 16 : per <= 32 ? 32 : 64;
       const long wgs = (long)T * n_kv * ((per + rows_wg - 1) / rows_wg);
       const long max_tiles = ((long)block_tables.size(1) * bs + 31) / 32;
       n_part = (int)std::min<long>(std::min<long>(32, (max_tiles + 1) / 2),
-                                   std::max<long>(1, 256 / wgs));
+                                   std::max<long>(1, 1024 / wgs));
       n_part = std::max(n_part, 1);
+      // tuning knob: fixed partition count (1..32)
+      if (const char* e = std::getenv("XLLM_CAPPED_PARTS"))
+        n_part = std::min(32, std::max(1, std::atoi(e)));
     }
     if (n_part > 1) {
       ws_acc = torch::empty({(long)T * heads * n_part, (long)Dv}, out.options());
@@ -703,6 +754,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_combine", &moe_combine);
   m.def("streams_mix_norm", &streams_mix_norm);
   m.def("streams_update", &streams_update);
+  m.def("streams_update_mix_norm", &streams_update_mix_norm);
   m.def("relu_sq", &relu_sq);
   m.def("softcap", &softcap);
   m.def("short_conv", &short_conv);

@@ -17,12 +17,15 @@
 // ctx_len == 0 starts from zero whatever its slot held before; slot < 0 runs
 // from zero and stores nothing.
 //
-// Prompt chunks: one workgroup per (sequence, head, 16 columns of Dv); thread
-// (j, r) owns rows r, r+16, ... of column j; a 16-lane shuffle sums a token's
-// output. Long chunks run piece-parallel: every piece builds its own state
+// Prompt chunks: one workgroup per (sequence, head, 16*CPT columns of Dv);
+// thread (j, r) owns rows r, r+16, ... of CPT neighbouring columns (CPT = 4
+// for wide values: a key/query/decay value read from LDS then feeds 8 FMAs);
+// a 16-lane shuffle sums a token's output. Long chunks run piece-parallel: every piece builds its own state
 // from zero together with the product of its decays, a scan turns these into
 // the state before each piece, a second pass writes the outputs. Decode: one
 // workgroup per (sequence, head) streams the state as whole rows.
+#include <cstdlib>
+
 #include "hybrid_common.h"
 
 namespace xllm {
@@ -30,8 +33,8 @@ namespace hyb {
 
 constexpr int GR_SSM = 0;
 constexpr int GR_GLA = 1;
-constexpr int GR_VS = 16;      // value columns per workgroup
-constexpr int GR_R = 16;       // row groups (threads per column)
+constexpr int GR_CG = 16;      // column groups per workgroup
+constexpr int GR_R = 16;       // row groups (threads per column group)
 constexpr int GR_TC = 16;      // tokens staged per LDS fill
 constexpr int GR_MAXM = 16;    // D <= GR_R * GR_MAXM = 256
 
@@ -67,13 +70,14 @@ XLLM_DEV void gr_stage_row(const GRArgs<T>& A, long row, int h, int i,
   }
 }
 
-template <typename T, int KIND>
+template <typename T, int KIND, int CPT>
 __global__ void __launch_bounds__(256) gated_recurrence_kernel(
     float* __restrict__ out, GRArgs<T> A, float* __restrict__ state,
     const int* __restrict__ slots, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int mode, int chunk, int max_chunks,
     float* __restrict__ ws, float* __restrict__ wa) {
   extern __shared__ float smem[];
+  constexpr int VS = GR_CG * CPT;         // value columns per workgroup
   const int D = A.D, Dv = A.Dv, heads = A.heads;
   const int Dd = (KIND == GR_SSM) ? 1 : D;
   float* qs = smem;                       // [TC][D]
@@ -88,11 +92,10 @@ __global__ void __launch_bounds__(256) gated_recurrence_kernel(
   // mode 2: the same tokens starting from ws[s*max_chunks + c] (as the scan
   //         left it), outputs written, no state out
   const int s = blockIdx.x / max_chunks, cidx = blockIdx.x % max_chunks;
-  const int h = blockIdx.y, v0 = blockIdx.z * GR_VS;
+  const int h = blockIdx.y, v0 = blockIdx.z * VS;
   const int tid = threadIdx.x;
   const int j = tid / GR_R, r = tid % GR_R;
-  const int col = v0 + j;
-  const bool col_ok = col < Dv;
+  const int col = v0 + j * CPT;           // first of this thread's columns
   int t0 = cu_q ? cu_q[s] : s;
   int t1 = cu_q ? cu_q[s + 1] : s + 1;
   if (mode != 0) {
@@ -103,9 +106,13 @@ __global__ void __launch_bounds__(256) gated_recurrence_kernel(
   const int slot = slots[s];
   const int M = (D + GR_R - 1) / GR_R;
 
-  float S[GR_MAXM], P[GR_MAXM];
+  float S[GR_MAXM][CPT], P[GR_MAXM];
 #pragma unroll
-  for (int m = 0; m < GR_MAXM; ++m) { S[m] = 0.f; P[m] = 1.f; }
+  for (int m = 0; m < GR_MAXM; ++m) {
+    P[m] = 1.f;
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) S[m][c] = 0.f;
+  }
   float* sp = (slot >= 0)
       ? state + (((long)slot * heads + h) * D) * (long)Dv : nullptr;
   bool load = sp && ctx_lens[s] > 0;
@@ -113,11 +120,23 @@ __global__ void __launch_bounds__(256) gated_recurrence_kernel(
     sp = ws + ((((long)s * max_chunks + cidx) * heads + h) * D) * (long)Dv;
     load = mode == 2;
   }
-  if (load && col_ok) {
+  const bool vec = CPT == 4 && (Dv & 3) == 0 && col + 3 < Dv;
+  if (load) {
 #pragma unroll
     for (int m = 0; m < GR_MAXM; ++m) {
       const int i = r + GR_R * m;
-      if (m < M && i < D) S[m] = sp[(long)i * Dv + col];
+      if (m < M && i < D) {
+        if (vec) {
+          const float4 x = *reinterpret_cast<const float4*>(
+              sp + (long)i * Dv + col);
+          S[m][0] = x.x; S[m][CPT > 1 ? 1 : 0] = x.y;
+          S[m][CPT > 2 ? 2 : 0] = x.z; S[m][CPT > 3 ? 3 : 0] = x.w;
+        } else {
+#pragma unroll
+          for (int c = 0; c < CPT; ++c)
+            if (col + c < Dv) S[m][c] = sp[(long)i * Dv + col + c];
+        }
+      }
     }
   }
   float dt_bias = 0.f, negA = 0.f, skip = 0.f;
@@ -146,38 +165,61 @@ __global__ void __launch_bounds__(256) gated_recurrence_kernel(
       gr_stage_row<T, KIND>(A, row, h, i, dt, qs + idx, ks + idx,
                             as + (KIND == GR_SSM ? 0 : idx));
     }
-    for (int idx = tid; idx < nt * GR_VS; idx += 256) {
-      const int tt = idx / GR_VS, jj = idx - tt * GR_VS;
+    for (int idx = tid; idx < nt * VS; idx += 256) {
+      const int tt = idx / VS, jj = idx - tt * VS;
       const long row = tb + tt;
       vs[idx] = (v0 + jj < Dv)
           ? IO<T>::ld(A.v + row * A.v_stride + h * Dv + v0 + jj) : 0.f;
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float vj = vs[tt * GR_VS + j];
-      float o = 0.f;
+      float vj[CPT], o[CPT];
+#pragma unroll
+      for (int c = 0; c < CPT; ++c) {
+        vj[c] = vs[tt * VS + j * CPT + c];
+        o[c] = 0.f;
+      }
 #pragma unroll
       for (int m = 0; m < GR_MAXM; ++m) {
         const int i = r + GR_R * m;
         if (m < M && i < D) {
           const float a = (KIND == GR_SSM) ? as[tt] : as[tt * D + i];
-          S[m] = a * S[m] + ks[tt * D + i] * vj;
-          o += S[m] * qs[tt * D + i];
+          const float kk = ks[tt * D + i], qq = qs[tt * D + i];
+#pragma unroll
+          for (int c = 0; c < CPT; ++c) {
+            S[m][c] = a * S[m][c] + kk * vj[c];
+            o[c] += S[m][c] * qq;
+          }
           if (mode == 1) P[m] *= a;
         }
       }
       if (mode != 1) {
-        o = group_reduce_sum<GR_R>(o);
-        if (r == 0 && col_ok)
-          out[((long)(tb + tt) * heads + h) * Dv + col] = o + skip * vj;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) o[c] = group_reduce_sum<GR_R>(o[c]);
+        if (r == 0) {
+          float* op = out + ((long)(tb + tt) * heads + h) * Dv + col;
+#pragma unroll
+          for (int c = 0; c < CPT; ++c)
+            if (col + c < Dv) op[c] = o[c] + skip * vj[c];
+        }
       }
     }
   }
-  if (sp && mode != 2 && col_ok) {
+  if (sp && mode != 2) {
 #pragma unroll
     for (int m = 0; m < GR_MAXM; ++m) {
       const int i = r + GR_R * m;
-      if (m < M && i < D) sp[(long)i * Dv + col] = S[m];
+      if (m < M && i < D) {
+        if (vec) {
+          *reinterpret_cast<float4*>(sp + (long)i * Dv + col) = make_float4(
+              S[m][0], S[m][CPT > 1 ? 1 : 0], S[m][CPT > 2 ? 2 : 0],
+              S[m][CPT > 3 ? 3 : 0]);
+        } else {
+#pragma unroll
+          for (int c = 0; c < CPT; ++c)
+            if (col + c < Dv) sp[(long)i * Dv + col + c] = S[m][c];
+        }
+      }
     }
   }
   if (mode == 1 && j == 0 && v0 == 0) {
@@ -274,6 +316,38 @@ __global__ void __launch_bounds__(256) gated_recurrence_decode_kernel(
   }
 }
 
+template <typename T, int KIND, int CPT>
+void launch_gated_recurrence_cpt(float* out, const GRArgs<T>& A, float* state,
+                                 const int* slots, const int* cu_q,
+                                 const int* ctx_lens, int n_seqs, int chunk,
+                                 int max_chunks, float* ws, float* wa,
+                                 hipStream_t st) {
+  const int D = A.D, Dv = A.Dv, heads = A.heads;
+  const int Dd = (KIND == GR_SSM) ? 1 : D;
+  constexpr int VS = GR_CG * CPT;
+  const size_t lds = (size_t)(2 * GR_TC * D + GR_TC * (KIND == GR_SSM ? 2 : D)
+                              + GR_TC * VS) * sizeof(float);
+  const int vz = (Dv + VS - 1) / VS;
+  if (ws == nullptr || max_chunks <= 1) {
+    hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND, CPT>),
+                       dim3(n_seqs, heads, vz), dim3(256), lds, st, out, A,
+                       state, slots, cu_q, ctx_lens, 0, 0, 1, nullptr, nullptr);
+    return;
+  }
+  dim3 grid(n_seqs * max_chunks, heads, vz);
+  hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND, CPT>), grid, dim3(256),
+                     lds, st, out, A, state, slots, cu_q, ctx_lens, 1, chunk,
+                     max_chunks, ws, wa);
+  const long per_seq = (long)heads * D * Dv;
+  hipLaunchKernelGGL(gated_recurrence_scan_kernel,
+                     dim3((unsigned)((per_seq + 255) / 256), n_seqs),
+                     dim3(256), 0, st, ws, wa, state, slots, cu_q, ctx_lens,
+                     heads, D, Dv, Dd, chunk, max_chunks);
+  hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND, CPT>), grid, dim3(256),
+                     lds, st, out, A, state, slots, cu_q, ctx_lens, 2, chunk,
+                     max_chunks, ws, wa);
+}
+
 template <typename T, int KIND>
 void launch_gated_recurrence_kind(float* out, const GRArgs<T>& A, float* state,
                                   const int* slots, const int* cu_q,
@@ -281,10 +355,6 @@ void launch_gated_recurrence_kind(float* out, const GRArgs<T>& A, float* state,
                                   int max_chunks, float* ws, float* wa,
                                   hipStream_t st) {
   const int D = A.D, Dv = A.Dv, heads = A.heads;
-  const int Dd = (KIND == GR_SSM) ? 1 : D;
-  const size_t lds = (size_t)(2 * GR_TC * D + GR_TC * (KIND == GR_SSM ? 2 : D)
-                              + GR_TC * GR_VS) * sizeof(float);
-  const int vz = (Dv + GR_VS - 1) / GR_VS;
   if (cu_q == nullptr && Dv % 4 == 0 && Dv <= 1024) {
     const int RG = 256 / (Dv / 4);
     const size_t l2 =
@@ -296,24 +366,19 @@ void launch_gated_recurrence_kind(float* out, const GRArgs<T>& A, float* state,
       return;
     }
   }
-  if (ws == nullptr || max_chunks <= 1) {
-    hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND>),
-                       dim3(n_seqs, heads, vz), dim3(256), lds, st, out, A,
-                       state, slots, cu_q, ctx_lens, 0, 0, 1, nullptr, nullptr);
-    return;
-  }
-  dim3 grid(n_seqs * max_chunks, heads, vz);
-  hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND>), grid, dim3(256), lds,
-                     st, out, A, state, slots, cu_q, ctx_lens, 1, chunk,
-                     max_chunks, ws, wa);
-  const long per_seq = (long)heads * D * Dv;
-  hipLaunchKernelGGL(gated_recurrence_scan_kernel,
-                     dim3((unsigned)((per_seq + 255) / 256), n_seqs),
-                     dim3(256), 0, st, ws, wa, state, slots, cu_q, ctx_lens,
-                     heads, D, Dv, Dd, chunk, max_chunks);
-  hipLaunchKernelGGL((gated_recurrence_kernel<T, KIND>), grid, dim3(256), lds,
-                     st, out, A, state, slots, cu_q, ctx_lens, 2, chunk,
-                     max_chunks, ws, wa);
+  // wide values and enough workgroups: four columns per thread (fewer LDS
+  // reads per FMA). XLLM_RECURRENCE_COLS=1|4 fixes the choice (tuning knob).
+  bool wide = Dv >= 48 &&
+      (long)n_seqs * max_chunks * heads * ((Dv + 63) / 64) >= 512;
+  if (const char* e = std::getenv("XLLM_RECURRENCE_COLS")) wide = e[0] == '4';
+  if (wide)
+    launch_gated_recurrence_cpt<T, KIND, 4>(out, A, state, slots, cu_q,
+                                            ctx_lens, n_seqs, chunk,
+                                            max_chunks, ws, wa, st);
+  else
+    launch_gated_recurrence_cpt<T, KIND, 1>(out, A, state, slots, cu_q,
+                                            ctx_lens, n_seqs, chunk,
+                                            max_chunks, ws, wa, st);
 }
 
 template <typename T>

@@ -87,6 +87,64 @@ __global__ void streams_update_kernel(
   }
 }
 
+// The write of one sublayer fused with the read of the next: a token's streams
+// are updated in place and the next sublayer's normed input is produced from
+// the new values in the same pass (one workgroup per token).
+template <typename T>
+__global__ void __launch_bounds__(256) streams_update_mix_norm_kernel(
+    T* __restrict__ out, float* __restrict__ x, const float* __restrict__ mix,
+    const float* __restrict__ w_out, const T* __restrict__ y1, float a1,
+    const T* __restrict__ y2, float a2, const float* __restrict__ w_in,
+    const float* __restrict__ g, const float* __restrict__ b, float eps, int S,
+    int W) {
+  extern __shared__ float u[];             // [W]
+  __shared__ float tmp[16];
+  __shared__ float m[MAX_STREAMS * MAX_STREAMS + 2 * MAX_STREAMS];
+  const int tid = threadIdx.x;
+  if (tid < S * S) m[tid] = mix ? mix[tid] : ((tid / S == tid % S) ? 1.f : 0.f);
+  if (tid < S) {
+    m[MAX_STREAMS * MAX_STREAMS + tid] = w_out ? w_out[tid] : 1.f;
+    m[MAX_STREAMS * MAX_STREAMS + MAX_STREAMS + tid] = w_in ? w_in[tid] : 1.f;
+  }
+  __syncthreads();
+  const long t = blockIdx.x;
+  float* xr = x + t * (long)S * W;
+  float sum = 0.f;
+  for (int c = tid; c < W; c += blockDim.x) {
+    float y = a1 * IO<T>::ld(y1 + t * (long)W + c);
+    if (y2) y += a2 * IO<T>::ld(y2 + t * (long)W + c);
+    float old[MAX_STREAMS];
+#pragma unroll
+    for (int s = 0; s < MAX_STREAMS; ++s)
+      if (s < S) old[s] = xr[(long)s * W + c];
+    float a = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAX_STREAMS; ++j) {
+      if (j < S) {
+        float acc = m[MAX_STREAMS * MAX_STREAMS + j] * y;
+#pragma unroll
+        for (int s = 0; s < MAX_STREAMS; ++s)
+          if (s < S) acc += m[s * S + j] * old[s];
+        xr[(long)j * W + c] = acc;
+        a += m[MAX_STREAMS * MAX_STREAMS + MAX_STREAMS + j] * acc;
+      }
+    }
+    u[c] = a;
+    sum += a;
+  }
+  const float mean = block_reduce_sum(sum, tmp) / (float)W;
+  float ss = 0.f;
+  for (int c = tid; c < W; c += blockDim.x) {
+    const float d = u[c] - mean;
+    ss += d * d;
+  }
+  __syncthreads();
+  const float var = block_reduce_sum(ss, tmp) / (float)W;
+  const float rs = 1.0f / sqrtf(var + eps);
+  for (int c = tid; c < W; c += blockDim.x)
+    IO<T>::st(out + t * (long)W + c, (u[c] - mean) * rs * g[c] + b[c]);
+}
+
 // x <- max(x, 0)^2 in place
 template <typename T>
 __global__ void relu_sq_kernel(T* __restrict__ x, long n) {
@@ -130,6 +188,17 @@ void launch_streams_update(float* x, const float* mix, const float* w_out,
                      S, W);
 }
 template <typename T>
+void launch_streams_update_mix_norm(T* out, float* x, const float* mix,
+                                    const float* w_out, const T* y1, float a1,
+                                    const T* y2, float a2, const float* w_in,
+                                    const float* g, const float* b, float eps,
+                                    int tokens, int S, int W, hipStream_t st) {
+  if (tokens == 0) return;
+  hipLaunchKernelGGL((streams_update_mix_norm_kernel<T>), dim3(tokens),
+                     dim3(256), (size_t)W * sizeof(float), st, out, x, mix,
+                     w_out, y1, a1, y2, a2, w_in, g, b, eps, S, W);
+}
+template <typename T>
 void launch_relu_sq(T* x, long n, hipStream_t st) {
   if (n == 0) return;
   hipLaunchKernelGGL((relu_sq_kernel<T>), dim3(blocks_for(n)), dim3(256), 0,
@@ -150,6 +219,10 @@ void launch_softcap(float* out, const T* x, float cap, long n,
   template void launch_streams_update<T>(float*, const float*, const float*,  \
                                          const T*, float, const T*, float,    \
                                          long, int, int, hipStream_t);        \
+  template void launch_streams_update_mix_norm<T>(                            \
+      T*, float*, const float*, const float*, const T*, float, const T*,      \
+      float, const float*, const float*, const float*, float, int, int, int,  \
+      hipStream_t);                                                           \
   template void launch_relu_sq<T>(T*, long, hipStream_t);                     \
   template void launch_softcap<T>(float*, const T*, float, long, hipStream_t);
 INST_STREAMS(float)

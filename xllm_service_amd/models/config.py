@@ -283,6 +283,46 @@ PRESETS.update({
 })
 
 
+def _dunusun_preset(name, width, n_layers, vocab=32000, every_attn=4,
+                    streams=2, head=128, state=128, loop=None):
+    """Synthetic Dunusun stacks for benchmarks: three selective state space
+    layers per parallel (attention + gated linear attention) layer, a dense
+    feed-forward of 1.5 x width in every layer."""
+    layers = []
+    mlp = dict(kind="dense", ff=3 * width // 2)
+    for i in range(n_layers):
+        if i % every_attn == every_attn - 1:
+            heads = max(width // head, 1)
+            left = dict(heads=heads, kv_heads=max(heads // 4, 1), dim=head,
+                        vdim=head, conv=4, scale=head ** -0.5, softcap=50.0,
+                        rot=dict(base=10000.0, dims=head // 2))
+            right = dict(heads=max(heads // 4, 1), dim=head, vdim=head,
+                         tau=16.0, rank=32)
+            layers.append(dict(type="parallel", mlp=mlp, mixer=dict(
+                left=left, right=right, left_scale=1.0, right_scale=1.0)))
+        else:
+            sh = max(width // (head // 2), 1)
+            layers.append(dict(type="mamba2", mlp=mlp, mixer=dict(
+                heads=sh, vdim=head // 2, state=state,
+                groups=max(sh // 4, 1), norm_groups=max(sh // 4, 1), conv=4)))
+    d = dict(architecture="Dunusun", vocab=vocab, width=width, layers=layers,
+             norm=dict(eps=1e-6), streams=streams, logit_softcap=30.0)
+    if loop:
+        d["loop"] = dict(start=loop[0], stop=loop[1], times=loop[2])
+    return dunusun_from_dict(d, name=name)
+
+
+PRESETS.update({
+    # CPU-test sized stack (the second layer runs twice)
+    "dunusun-tiny": _dunusun_preset("dunusun-tiny", 64, 3, vocab=256,
+                                    every_attn=2, head=16, state=8,
+                                    loop=(1, 2, 2)),
+    # bench stacks at the width of real deployments (random weights)
+    "dunusun-2k": _dunusun_preset("dunusun-2k", 2048, 8),
+    "dunusun-4k": _dunusun_preset("dunusun-4k", 4096, 8),
+})
+
+
 def get_config(name: str) -> ModelConfig:
     if os.path.isdir(name):
         return load_model_dir(name)

@@ -58,11 +58,14 @@ class StreamPort(nn.Module):
         return hops.streams_mix_norm(x, self.w_in if self.mixed else None,
                                      self.norm_w, self.norm_b, self.eps, dtype)
 
-    def write(self, x, y1, a1=1.0, y2=None, a2=0.0):
-        if self.mixed:
-            return hops.streams_update_(x, self.mix, self.w_out, y1, a1, y2,
-                                        a2)
-        return hops.streams_update_(x, None, None, y1, a1, y2, a2)
+    def write_then_read(self, x, nxt: "StreamPort", y1, a1=1.0, y2=None,
+                        a2=0.0):
+        """This sublayer's write and the next port's read in one pass over
+        the streams; returns the next sublayer's normed input."""
+        mix, w_out = (self.mix, self.w_out) if self.mixed else (None, None)
+        return hops.streams_update_mix_norm_(
+            x, mix, w_out, y1, a1, y2, a2, nxt.w_in if nxt.mixed else None,
+            nxt.norm_w, nxt.norm_b, nxt.eps)
 
 
 class DunusunLayer(nn.Module):
@@ -96,19 +99,21 @@ class DunusunLayer(nn.Module):
             self.down = nn.Parameter(torch.empty(W, lc.mlp["ff"], dtype=dtype))
             self.port2 = StreamPort(W, cfg.streams, eps)
 
-    def forward(self, x, positions, cache, meta, aux):
-        h = self.port1.read(x, self.dtype)
+    def forward(self, x, h, positions, cache, meta, aux, next_port):
+        """x: the streams (updated in place); h: this layer's normed mixer
+        input, read by the previous layer's last write. Returns the streams
+        and the normed input of whatever follows (`next_port`)."""
         y = self.mixer(F.linear(h, self.in_proj), positions, cache, meta, aux)
+        after = self.port2 if self.ff else next_port
         if isinstance(y, tuple):
             a1, a2 = self.mixer.scales
-            self.port1.write(x, y[0], a1, y[1], a2)
+            h = self.port1.write_then_read(x, after, y[0], a1, y[1], a2)
         else:
-            self.port1.write(x, y)
+            h = self.port1.write_then_read(x, after, y)
         if self.ff:
-            h = self.port2.read(x, self.dtype)
             y = F.linear(hops.relu_sq_(F.linear(h, self.up)), self.down)
-            self.port2.write(x, y)
-        return x
+            h = self.port2.write_then_read(x, next_port, y)
+        return x, h
 
 
 class DunusunForCausalLM(nn.Module):
@@ -124,7 +129,8 @@ class DunusunForCausalLM(nn.Module):
         self.layers = nn.ModuleList(
             [DunusunLayer(cfg, i, ranks, dtype)
              for i in range(cfg.num_layers)])
-        self.final_norm, self.final_norm_b = _f32(W), _f32(W, fill=0.0)
+        # the read in front of the head: plain sum of the streams, normed
+        self.final = StreamPort(W, None, cfg.rms_eps)
         self.lm_head = nn.Parameter(torch.empty(cfg.vocab_size, W,
                                                 dtype=dtype))
         self.runs: List[int] = cfg.layer_runs
@@ -179,8 +185,8 @@ class DunusunForCausalLM(nn.Module):
                 put(port.mix, take(f"{p}hc{q}.mix"))
 
         put(self.embed.weight, take("embed"))
-        put(self.final_norm, take("final.norm"))
-        put(self.final_norm_b, take("final.norm.b"))
+        put(self.final.norm_w, take("final.norm"))
+        put(self.final.norm_b, take("final.norm.b"))
         put(self.lm_head, take("head"))
         for i, layer in enumerate(self.layers):
             p = f"l{i}."
@@ -230,7 +236,7 @@ class DunusunForCausalLM(nn.Module):
                             + 0.1 * randn(p.shape))
                 elif leaf == "w_in":
                     p.fill_(1.0 / p.shape[0])
-                elif leaf in ("norm_b", "final_norm_b", "conv_b", "dt_bias"):
+                elif leaf in ("norm_b", "conv_b", "dt_bias"):
                     p.zero_()
                 elif leaf == "A_log":
                     p.copy_(-1.0 + 0.5 * randn(p.shape))
@@ -255,11 +261,16 @@ class DunusunForCausalLM(nn.Module):
         aux = {}
         if meta.num_decode_tokens:
             aux["decode_ctx_lens"] = meta.decode_seq_lens - 1
+        if not self.runs:
+            return self.final.read(x, self.dtype)
+        # every write to the streams is fused with the read that follows it
+        h = self.layers[self.runs[0]].port1.read(x, self.dtype)
         for run, li in enumerate(self.runs):
-            x = self.layers[li](x, positions, kv_caches[run], meta, aux)
-        return hops.streams_mix_norm(x, None, self.final_norm,
-                                     self.final_norm_b, self.cfg.rms_eps,
-                                     self.dtype)
+            nxt = (self.layers[self.runs[run + 1]].port1
+                   if run + 1 < len(self.runs) else self.final)
+            x, h = self.layers[li](x, h, positions, kv_caches[run], meta, aux,
+                                   nxt)
+        return h
 
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
         logits = F.linear(hidden, self.lm_head)

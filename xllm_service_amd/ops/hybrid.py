@@ -173,6 +173,21 @@ def streams_update_(x, mix, w_out, y1, a1: float = 1.0, y2=None,
     return ref.streams_update(x, mix, w_out, y1, a1, y2, a2)
 
 
+def streams_update_mix_norm_(x, mix, w_out, y1, a1, y2, a2, w_in, g, b,
+                             eps: float):
+    """streams_update_ followed by streams_mix_norm of the new values (the
+    next sublayer's read) in one pass; returns the normed input in y1's
+    dtype."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], x.shape[2], dtype=y1.dtype,
+                          device=x.device)
+        _hyb().streams_update_mix_norm(out, x, mix, w_out, y1, a1, y2, a2,
+                                       w_in, g, b, eps)
+        return out
+    ref.streams_update(x, mix, w_out, y1, a1, y2, a2)
+    return ref.streams_mix_norm(x, w_in, g, b, eps, y1.dtype)
+
+
 def relu_sq_(x):
     if x.is_cuda:
         _hyb().relu_sq(x)
