@@ -55,6 +55,20 @@ def _variants():
             par_layer(heads=2, kv_heads=2, dim=8, vdim=16, conv=5, dims=2,
                       scale=0.5, softcap=1.5, r_heads=4, r_dim=8, r_vdim=4)],
                             loop=(1, 2, 3)),
+        # head widths of the matrix-core attention classes, value rows wide
+        # enough for four columns per thread, three query heads per group
+        "large": make_config(width=128, vocab=200, streams=3, eps=1e-6,
+                             layers=[
+            par_layer(heads=6, kv_heads=2, dim=64, vdim=128, conv=4, dims=32,
+                      base=10000.0, softcap=20.0, r_heads=2, r_dim=48,
+                      r_vdim=32, tau=16.0, rank=16, left_scale=0.8,
+                      right_scale=1.1, mlp=192),
+            ssm_layer(heads=4, vdim=64, state=32, groups=2, norm_groups=2,
+                      conv=3, mlp=192),
+            par_layer(heads=2, kv_heads=1, dim=128, vdim=64, conv=2, dims=128,
+                      base=500.0, softcap=None, r_heads=1, r_dim=64,
+                      r_vdim=64, tau=2.0, rank=8, mlp=None)],
+                             loop=(0, 2, 2), logit_softcap=30.0),
     }
 
 
@@ -115,7 +129,7 @@ def _run_portions(eng, rid, toks, cuts, end=True):
     return torch.cat(out)
 
 
-NAMES = ["mixed", "plain", "ones", "wide"]
+NAMES = ["mixed", "plain", "ones", "wide", "large"]
 
 
 @pytest.mark.parametrize("target", TARGETS)
@@ -172,7 +186,7 @@ def test_prefill_then_token_by_token(root, target, name):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("name", ["mixed", "wide"])
+@pytest.mark.parametrize("name", ["mixed", "wide", "large"])
 def test_portions_of_many_sizes(root, target, name):
     cfg, w, folder = _model(name, root)
     eng = _engine(folder, target)
@@ -280,6 +294,62 @@ def test_greedy_generation_through_scheduler(root, target, name):
             seq.append(tok)
     assert eng.block_manager.num_free == 32
     assert eng.state_manager.num_free == 2
+
+
+def test_preset_generates_through_the_engine():
+    """The named preset (random weights; its second layer runs twice)."""
+    eng = LLMEngine("dunusun-tiny", device="cpu", max_num_seqs=2,
+                    max_kv_blocks=16, max_model_len=128, swap_space_mb=0)
+    a = eng.generate([[1, 2, 3, 4, 5, 6, 7], [9, 8]],
+                     SamplingParams(max_tokens=4, ignore_eos=True))
+    b = eng.generate([[9, 8]], SamplingParams(max_tokens=4, ignore_eos=True))
+    assert [len(x) for x in a] == [4, 4] and a[1] == b[0]
+    assert eng.state_manager.num_free == 2
+
+
+def test_trace_replay_command(root, tmp_path):
+    """bin/trace_run on a model folder: steps on stdin, logits in files, a
+    pool of two slots and 128 tokens used by three requests in turn."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    cfg, w, folder = _model("plain", root)
+    toks = {k: _tokens(cfg, n, 60 + n) for k, n in (("a", 40), ("b", 9),
+                                                     ("c", 30))}
+    steps = [
+        dict(step=0, entries=[dict(id="a", tokens=toks["a"][:33], want=[0, 32]),
+                              dict(id="b", tokens=toks["b"][:8], want=[])],
+             end=[]),
+        dict(step=1, entries=[dict(id="a", tokens=toks["a"][33:34], want=[0]),
+                              dict(id="b", tokens=toks["b"][8:], want=[0])],
+             end=["b"]),
+        dict(step=2, entries=[dict(id="c", tokens=toks["c"][:2], want=[1])],
+             end=[]),
+        dict(step=3, entries=[dict(id="a", tokens=toks["a"][34:], want=[5]),
+                              dict(id="c", tokens=toks["c"][2:], want=[27])],
+             end=["a", "c"]),
+    ]
+    exe = os.path.join(os.path.dirname(os.path.dirname(
+        os.path.abspath(__file__))), "bin", "trace_run")
+    out = tmp_path / "out"
+    p = subprocess.run(
+        [sys.executable, exe, "--model", folder, "--dtype", "float32", "--out",
+         str(out), "--max-tokens", "128", "--slots", "2", "--device", "cpu"],
+        input="".join(json.dumps(x) + "\n" for x in steps), text=True,
+        capture_output=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.split("\n") if l.startswith("done")] == [
+        f"done {i}" for i in range(4)]
+    full = {k: o_forward(cfg, w, t)[0] for k, t in toks.items()}
+    want = {0: [full["a"][0], full["a"][32]], 1: [full["a"][33], full["b"][8]],
+            2: [full["c"][1]], 3: [full["a"][39], full["c"][29]]}
+    for i, rows in want.items():
+        got = torch.from_numpy(np.fromfile(out / f"{i}.f32", dtype="<f4")
+                               .reshape(len(rows), -1).copy())
+        _check(got, torch.stack(rows), ("cpu", torch.float32), i)
 
 
 def test_config_is_checked(tmp_path):

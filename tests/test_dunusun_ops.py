@@ -412,6 +412,7 @@ def test_attention_sizes_and_groups(target):
 @pytest.mark.parametrize("target", TARGETS)
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 128, 256), (2, 1, 128, 128),
                                       (2, 2, 256, 256), (40, 2, 64, 64),
+                                      (36, 1, 32, 64),
                                       (3, 1, 24, 136)])
 def test_attention_wide_heads(target, H, G, D, Dv):
     """Head widths of every size class of the matrix-core kernel, prompt

@@ -20,7 +20,7 @@
 // Prompt chunks: one workgroup per (sequence, head, 16*CPT columns of Dv);
 // thread (j, r) owns rows r, r+16, ... of CPT neighbouring columns (CPT = 4
 // for wide values: a key/query/decay value read from LDS then feeds 8 FMAs);
-// a 16-lane shuffle sums a token's output. Long chunks run piece-parallel: every piece builds its own state
+// a 16-lane DPP reduction sums a token's output. Long chunks run piece-parallel: every piece builds its own state
 // from zero together with the product of its decays, a scan turns these into
 // the state before each piece, a second pass writes the outputs. Decode: one
 // workgroup per (sequence, head) streams the state as whole rows.
@@ -37,6 +37,21 @@ constexpr int GR_CG = 16;      // column groups per workgroup
 constexpr int GR_R = 16;       // row groups (threads per column group)
 constexpr int GR_TC = 16;      // tokens staged per LDS fill
 constexpr int GR_MAXM = 16;    // D <= GR_R * GR_MAXM = 256
+
+// Sum over the 16 lanes of a DPP row, left in every lane: lane-crossing
+// inside the vector ALU (quad permutes, then the two mirror modes) instead of
+// four trips through the LDS crossbar.
+XLLM_DEV float row16_sum(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(
+      0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(
+      0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(
+      0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(
+      0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return v;
+}
 
 XLLM_DEV float softplusf_(float x) {
   return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x)));
@@ -195,7 +210,7 @@ __global__ void __launch_bounds__(256) gated_recurrence_kernel(
       }
       if (mode != 1) {
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) o[c] = group_reduce_sum<GR_R>(o[c]);
+        for (int c = 0; c < CPT; ++c) o[c] = row16_sum(o[c]);
         if (r == 0) {
           float* op = out + ((long)(tb + tt) * heads + h) * Dv + col;
 #pragma unroll
