@@ -1,6 +1,6 @@
 """The README deployment commands work as-is: `python -m ...master` and
 `python -m ...worker` as real subprocesses, speaking over the loopback
-(CPU, llama-tiny)."""
+(CPU; a dense-attention preset and a hybrid one with recurrent state)."""
 import json
 import os
 import socket
@@ -21,7 +21,8 @@ def _free_port():
 
 
 @pytest.mark.timeout(180)
-def test_master_and_worker_cli():
+@pytest.mark.parametrize("model", ["llama-tiny", "dunusun-tiny"])
+def test_master_and_worker_cli(model):
     http_port, rpc_port, reg_port = _free_port(), _free_port(), _free_port()
     env = dict(os.environ)
     procs = []
@@ -30,12 +31,12 @@ def test_master_and_worker_cli():
             [sys.executable, "-m", "xllm_service_amd.service.master",
              "--http-host", "127.0.0.1", "--http-port", str(http_port),
              "--rpc-port", str(rpc_port), "--registry-port", str(reg_port),
-             "--model-id", "llama-tiny", "--policy", "RR"],
+             "--model-id", model, "--policy", "RR"],
             cwd=ROOT, env=env, stdout=subprocess.PIPE,
             stderr=subprocess.STDOUT))
         procs.append(subprocess.Popen(
             [sys.executable, "-m", "xllm_service_amd.engine.worker",
-             "--name", "w0", "--type", "DEFAULT", "--model", "llama-tiny",
+             "--name", "w0", "--type", "DEFAULT", "--model", model,
              "--device", "cpu", "--registry-port", str(reg_port),
              "--seed", "0"],
             cwd=ROOT, env=env, stdout=subprocess.PIPE,
@@ -52,7 +53,7 @@ def test_master_and_worker_cli():
                     base + "/v1/completions", method="POST",
                     headers={"Content-Type": "application/json"},
                     data=json.dumps({
-                        "model": "llama-tiny", "prompt": [3, 4, 5],
+                        "model": model, "prompt": [3, 4, 5],
                         "max_tokens": 4, "temperature": 0.0,
                         "ignore_eos": True}).encode())
                 with urllib.request.urlopen(req, timeout=10) as r:
@@ -64,7 +65,7 @@ def test_master_and_worker_cli():
         assert body["usage"]["completion_tokens"] == 4
         with urllib.request.urlopen(base + "/v1/models", timeout=10) as r:
             models = json.loads(r.read())
-        assert models["data"][0]["id"] == "llama-tiny"
+        assert models["data"][0]["id"] == model
         with urllib.request.urlopen(base + "/metrics", timeout=10) as r:
             assert b"server_request_in_total" in r.read()
     finally:
