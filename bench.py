@@ -360,6 +360,15 @@ def _dunusun_kernels(size, device, T, batch, ctx):
     y = torch.randn(T, Wd, **bf)
     t = _time_gpu(lambda: hops.streams_update_(xs, mix, wi, y, 1.0, y, 1.0))
     out.append(("streams_update", t, T * Wd * (8 * S + 4) / t / 1e9, "GB/s"))
+    t = _time_gpu(lambda: hops.streams_update_mix_norm_(
+        xs, mix, wi, y, 1.0, y, 1.0, wi, w, w, 1e-6))
+    out.append(("streams_update_mix_norm (fused)", t,
+                T * Wd * (8 * S + 6) / t / 1e9, "GB/s"))
+    xsd, yd = xs[:batch].contiguous(), y[:batch].contiguous()
+    t = _time_gpu(lambda: hops.streams_update_mix_norm_(
+        xsd, mix, wi, yd, 1.0, yd, 1.0, wi, w, w, 1e-6))
+    out.append((f"streams_update_mix_norm, {batch} rows (decode)", t,
+                batch * Wd * (8 * S + 6) / t / 1e9, "GB/s"))
     x1 = torch.randn(T, Wd, **f32)
     t = _time_gpu(lambda: hops.group_rmsnorm(x1, w, 1e-6, pc.norm_groups,
                                              torch.bfloat16))

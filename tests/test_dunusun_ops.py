@@ -39,7 +39,7 @@ def _i32(x, dev):
 
 # ------------------------------------------------------------ residual streams
 @pytest.mark.parametrize("target", TARGETS)
-@pytest.mark.parametrize("S,W", [(1, 20), (3, 70), (8, 257)])
+@pytest.mark.parametrize("S,W", [(1, 20), (3, 70), (8, 257), (2, 1288)])
 def test_streams_read_and_write(target, S, W):
     dev, dt = target
     g = torch.Generator().manual_seed(S * 100 + W)

@@ -87,10 +87,36 @@ __global__ void streams_update_kernel(
   }
 }
 
+// four neighbouring values at once (16 B of fp32, 8 B of bf16)
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  static XLLM_DEV void ld(const float* p, float v[4]) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  static XLLM_DEV void st(float* p, const float v[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Quad<unsigned short> {
+  static XLLM_DEV void ld(const unsigned short* p, float v[4]) {
+    const ushort4_t x = *reinterpret_cast<const ushort4_t*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = bf16_to_f32(x.x[i]);
+  }
+  static XLLM_DEV void st(unsigned short* p, const float v[4]) {
+    ushort4_t x;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x.x[i] = f32_to_bf16(v[i]);
+    *reinterpret_cast<ushort4_t*>(p) = x;
+  }
+};
+
 // The write of one sublayer fused with the read of the next: a token's streams
 // are updated in place and the next sublayer's normed input is produced from
-// the new values in the same pass (one workgroup per token).
-template <typename T>
+// the new values in the same pass (one workgroup per token). V = 4: four
+// columns per thread and access (width a multiple of 4), V = 1: any width.
+template <typename T, int V>
 __global__ void __launch_bounds__(256) streams_update_mix_norm_kernel(
     T* __restrict__ out, float* __restrict__ x, const float* __restrict__ mix,
     const float* __restrict__ w_out, const T* __restrict__ y1, float a1,
@@ -110,39 +136,70 @@ __global__ void __launch_bounds__(256) streams_update_mix_norm_kernel(
   const long t = blockIdx.x;
   float* xr = x + t * (long)S * W;
   float sum = 0.f;
-  for (int c = tid; c < W; c += blockDim.x) {
-    float y = a1 * IO<T>::ld(y1 + t * (long)W + c);
-    if (y2) y += a2 * IO<T>::ld(y2 + t * (long)W + c);
-    float old[MAX_STREAMS];
+  for (int c = tid * V; c < W; c += blockDim.x * V) {
+    float y[V], yb[V], old[MAX_STREAMS][V], a[V];
+    if (V == 4) {
+      Quad<T>::ld(y1 + t * (long)W + c, y);
+      if (y2) Quad<T>::ld(y2 + t * (long)W + c, yb);
+    } else {
+      y[0] = IO<T>::ld(y1 + t * (long)W + c);
+      if (y2) yb[0] = IO<T>::ld(y2 + t * (long)W + c);
+    }
 #pragma unroll
-    for (int s = 0; s < MAX_STREAMS; ++s)
-      if (s < S) old[s] = xr[(long)s * W + c];
-    float a = 0.f;
+    for (int i = 0; i < V; ++i) {
+      y[i] = a1 * y[i] + (y2 ? a2 * yb[i] : 0.f);
+      a[i] = 0.f;
+    }
+#pragma unroll
+    for (int s = 0; s < MAX_STREAMS; ++s) {
+      if (s < S) {
+        if (V == 4) Quad<float>::ld(xr + (long)s * W + c, old[s]);
+        else old[s][0] = xr[(long)s * W + c];
+      }
+    }
 #pragma unroll
     for (int j = 0; j < MAX_STREAMS; ++j) {
       if (j < S) {
-        float acc = m[MAX_STREAMS * MAX_STREAMS + j] * y;
+        float acc[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+          acc[i] = m[MAX_STREAMS * MAX_STREAMS + j] * y[i];
 #pragma unroll
         for (int s = 0; s < MAX_STREAMS; ++s)
-          if (s < S) acc += m[s * S + j] * old[s];
-        xr[(long)j * W + c] = acc;
-        a += m[MAX_STREAMS * MAX_STREAMS + MAX_STREAMS + j] * acc;
+          if (s < S) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[i] += m[s * S + j] * old[s][i];
+          }
+        if (V == 4) Quad<float>::st(xr + (long)j * W + c, acc);
+        else xr[(long)j * W + c] = acc[0];
+#pragma unroll
+        for (int i = 0; i < V; ++i)
+          a[i] += m[MAX_STREAMS * MAX_STREAMS + MAX_STREAMS + j] * acc[i];
       }
     }
-    u[c] = a;
-    sum += a;
+#pragma unroll
+    for (int i = 0; i < V; ++i) { u[c + i] = a[i]; sum += a[i]; }
   }
   const float mean = block_reduce_sum(sum, tmp) / (float)W;
   float ss = 0.f;
-  for (int c = tid; c < W; c += blockDim.x) {
-    const float d = u[c] - mean;
-    ss += d * d;
+  for (int c = tid * V; c < W; c += blockDim.x * V) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = u[c + i] - mean;
+      ss += d * d;
+    }
   }
   __syncthreads();
   const float var = block_reduce_sum(ss, tmp) / (float)W;
   const float rs = 1.0f / sqrtf(var + eps);
-  for (int c = tid; c < W; c += blockDim.x)
-    IO<T>::st(out + t * (long)W + c, (u[c] - mean) * rs * g[c] + b[c]);
+  for (int c = tid * V; c < W; c += blockDim.x * V) {
+    float h[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i)
+      h[i] = (u[c + i] - mean) * rs * g[c + i] + b[c + i];
+    if (V == 4) Quad<T>::st(out + t * (long)W + c, h);
+    else IO<T>::st(out + t * (long)W + c, h[0]);
+  }
 }
 
 // x <- max(x, 0)^2 in place
@@ -194,9 +251,14 @@ void launch_streams_update_mix_norm(T* out, float* x, const float* mix,
                                     const float* g, const float* b, float eps,
                                     int tokens, int S, int W, hipStream_t st) {
   if (tokens == 0) return;
-  hipLaunchKernelGGL((streams_update_mix_norm_kernel<T>), dim3(tokens),
-                     dim3(256), (size_t)W * sizeof(float), st, out, x, mix,
-                     w_out, y1, a1, y2, a2, w_in, g, b, eps, S, W);
+  if (W % 4 == 0)
+    hipLaunchKernelGGL((streams_update_mix_norm_kernel<T, 4>), dim3(tokens),
+                       dim3(256), (size_t)W * sizeof(float), st, out, x, mix,
+                       w_out, y1, a1, y2, a2, w_in, g, b, eps, S, W);
+  else
+    hipLaunchKernelGGL((streams_update_mix_norm_kernel<T, 1>), dim3(tokens),
+                       dim3(256), (size_t)W * sizeof(float), st, out, x, mix,
+                       w_out, y1, a1, y2, a2, w_in, g, b, eps, S, W);
 }
 template <typename T>
 void launch_relu_sq(T* x, long n, hipStream_t st) {
