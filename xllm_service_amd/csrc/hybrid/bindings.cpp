@@ -631,6 +631,9 @@ void gated_recurrence(long kind, Tensor out, Tensor q, Tensor k, Tensor v,
   if (cu != nullptr) {
     const long bound = max_q_len > 0 ? std::min<long>(max_q_len, T) : T;
     const long per_seq = (long)H * D * Dv * 4;
+    // tuning knob: piece length of the piece-parallel passes
+    if (const char* e = std::getenv("XLLM_RECURRENCE_CHUNK"))
+      chunk = std::min(1024, std::max(16, std::atoi(e)));
     // few heads: shorter pieces, so that the piece-parallel passes still
     // fill the chip
     while (chunk > 32 &&
