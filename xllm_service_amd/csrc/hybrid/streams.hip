@@ -9,7 +9,9 @@
 //   x[t,j] = sum_s mix[s, j] * x[t, s] + w_out[j] * (a1 * y1 + a2 * y2)
 //
 // With S = 1, w_in = mix = w_out = 1 this is the plain pre-norm residual.
-// One workgroup per token for the read; the write is elementwise.
+// One workgroup per token for the read; the write alone is elementwise; the
+// model's steady state is the fused kernel (a write and the next read in one
+// pass over the token's streams).
 #include "hybrid_common.h"
 
 namespace xllm {

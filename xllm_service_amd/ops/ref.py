@@ -363,9 +363,8 @@ def short_conv(x, w, bias, state, state_off, slots, cu_q, ctx_lens, heads, hd,
     if act_silu:
         out = torch.nn.functional.silu(out)
     if rot_dims:
-        o3 = out.view(T, heads, hd).to(x.dtype)
-        out = rope_interleaved(o3, positions, inv_freq, 1.0, rot_dims) \
-            .reshape(T, C)
+        out = rope_interleaved(out.view(T, heads, hd), positions, inv_freq,
+                               1.0, rot_dims).reshape(T, C)
     return out.to(x.dtype)
 
 
